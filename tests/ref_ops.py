@@ -25,21 +25,98 @@ def embed_rows(tokens, table, scale):
     return table[tokens.long()].float() * scale
 
 
-def _norm(x, gain, eps):
+def _norm(x, gain, eps, groups=1):
     x = x.float()
-    return x * torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps) * gain
+    parts = x.reshape(x.shape[0], groups, -1)
+    parts = parts * torch.rsqrt((parts * parts).mean(dim=-1, keepdim=True) + eps)
+    return parts.reshape(x.shape) * gain
 
 
-def rms_norm(x, gain, eps, out_dtype):
-    return _norm(x, gain, eps).to(out_dtype)
+def rms_norm(x, gain, eps, out_dtype, groups=1):
+    return _norm(x, gain, eps, groups).to(out_dtype)
 
 
-def add_rms_norm(stream, rows, gain_post, eps_post, gain_next, eps_next, out_dtype):
-    t = rows.float() if gain_post is None else _norm(rows, gain_post, eps_post)
+def add_rms_norm(stream, rows, gain_post, eps_post, gain_next, eps_next, out_dtype, groups=1):
+    t = rows.float() if gain_post is None else _norm(rows, gain_post, eps_post, groups)
     stream += t
     if gain_next is None:
         return None
-    return _norm(stream, gain_next, eps_next).to(out_dtype)
+    return _norm(stream, gain_next, eps_next, groups).to(out_dtype)
+
+
+def scale_rows(x, scale):
+    x *= scale
+
+
+def causal_conv(stream, w, state, slot_ids, cu_rows, row_seq, out_dtype, residual=True, one_row_each=False):
+    """out_t = (x_t) + sum_j w[:, j] x_(t - taps + 1 + j); rows before the step come from state[slot] ([taps - 1, D],
+    oldest first), which then takes the last taps - 1 rows of (state, step)."""
+    taps = w.shape[1]
+    out = torch.empty(stream.shape, dtype=torch.float32, device=stream.device)
+    for i in range(len(cu_rows) - 1):
+        a, b, slot = int(cu_rows[i]), int(cu_rows[i + 1]), int(slot_ids[i])
+        hist = stream[a:b] if taps == 1 else torch.cat([state[slot], stream[a:b]])
+        acc = stream[a:b].clone() if residual else torch.zeros_like(stream[a:b])
+        for j in range(taps):
+            acc += w[:, j] * hist[j:j + (b - a)]
+        out[a:b] = acc
+        if taps > 1:
+            state[slot] = hist[hist.shape[0] - (taps - 1):].clone()
+    return out.to(out_dtype)
+
+
+def latent_prepare(proj, H, dn, dr, R, gain, eps, inv_freq, rot, row_seq, row_pos, new_len, table, pool, rows_cap,
+                   own=True, out_dtype=None):
+    """proj [M, H (dr + dn) (+ dr + R)]: per head [rotated | unrotated] query parts, then [key part | latent].
+    Returns q [M, H (dr + R)] with every head's first dr elements set (the rotated query part; the rest is for
+    `head_linear`), and the step's rows [rope(key part) | rmsnorm(latent) * gain] (None when own is false), which are
+    also written into the cache."""
+    m = proj.shape[0]
+    out_dtype = out_dtype or proj.dtype
+    q = torch.zeros((m, H, dr + R), dtype=out_dtype, device=proj.device)
+    qr = proj[:, :H * (dr + dn)].float().reshape(m, H, dr + dn)[:, :, :dr]
+    q[:, :, :dr] = _rotate(qr, row_pos, inv_freq, rot).to(out_dtype)
+    mine = None
+    if own:
+        tail = proj[:, H * (dr + dn):].float()
+        r = _rotate(tail[:, None, :dr], row_pos, inv_freq, rot)[:, 0]
+        c = tail[:, dr:]
+        c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * gain
+        mine = torch.cat([r, c], dim=-1).to(out_dtype)
+        _cache_rows(mine, mine, row_seq, row_pos, new_len, table, pool, pool, rows_cap)
+    return q.reshape(m, H * (dr + R)), mine
+
+
+def head_linear(x, w, out=None):
+    """x [M, H, K] (any strides), w [H, N, K] -> out [M, H, N] (a view to fill, or a new tensor of x's dtype)."""
+    y = torch.einsum("mhk,hnk->mhn", x.float(), w.float())
+    if out is None:
+        return y.to(x.dtype).contiguous()
+    out.copy_(y.to(out.dtype))
+    return out
+
+
+def route_top(logits, top, renormalize=False):
+    s = torch.softmax(logits.float(), dim=-1)
+    order = torch.argsort(-s, dim=-1, stable=True)[:, :top]
+    w = torch.gather(s, 1, order)
+    if renormalize:
+        w = w / w.sum(-1, keepdim=True)
+    return order.to(torch.int32), w
+
+
+def expert_ffn(x, chosen, weights, w_gate_up, w_down, limit, alpha, shift):
+    """fp32 [M, D]: sum over a token's chosen experts, in the order they were chosen, of weight * expert(x)."""
+    m, ff = x.shape[0], w_gate_up.shape[1] // 2
+    out = torch.zeros((m, w_down.shape[1]), dtype=torch.float32, device=x.device)
+    for k in range(chosen.shape[1]):
+        for r in range(m):
+            e = int(chosen[r, k])
+            gu = w_gate_up[e].float() @ x[r].float()
+            g, u = torch.clamp(gu[:ff], max=limit), torch.clamp(gu[ff:], -limit, limit)
+            y = (g * torch.sigmoid(alpha * g) * (u + shift)).to(x.dtype).float()
+            out[r] += weights[r, k] * (w_down[e].float() @ y)
+    return out
 
 
 def linear(x, w, out_dtype, softcap=None, defer=False, bias=None):

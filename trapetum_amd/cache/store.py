@@ -117,7 +117,9 @@ class ModelCache:
     max_context: longest single sequence.
     """
 
-    def __init__(self, entry_specs, max_tokens, max_context, max_slots, page_size, dtype, device):
+    def __init__(self, entry_specs, max_tokens, max_context, max_slots, page_size, dtype, device, entry_states=None):
+        """entry_states: for every schedule entry, {name: StateSpec} of states it keeps beside its mixer's cache (what a
+        block's own operations carry from step to step); a run that reads another run's cache still has its own."""
         if page_size <= 0 or page_size % 16:
             raise CacheError(f"page size {page_size} must be a positive multiple of 16")
         self.page_size = page_size
@@ -146,11 +148,29 @@ class ModelCache:
                 raise CacheError(f"schedule entry declares an unknown cache need: {spec!r}")
             for i, entry in enumerate(entries):
                 self._site_of[entry] = CacheSite(spec, gi, i, g)
+        self._named_states = {}
+        keyed = {}
+        for entry, states in enumerate(entry_states or ()):
+            for name, spec in (states or {}).items():
+                if not isinstance(spec, StateSpec):
+                    raise CacheError(f"schedule entry {entry} declares state '{name}' as {spec!r}: not a StateSpec")
+                keyed.setdefault(spec, []).append((entry, name))
+        for spec, owners in keyed.items():
+            g = _StateGroup(spec, [e for e, _ in owners], max_slots, dtype, device)
+            self.state_groups.append(g)
+            for i, owner in enumerate(owners):
+                self._named_states[owner] = g.tensor[i]
         self.book = SlotBook(max_slots, [g.pages for g in self.token_groups], max_context)
 
     # --- what parts use -------------------------------------------------------------
     def site(self, entry):
         return self._site_of.get(entry)
+
+    def entry_state(self, entry, name):
+        """A state the entry declared by name: [slots + 1, *shape], zero for a slot that was just taken."""
+        if (entry, name) not in self._named_states:
+            raise CacheError(f"schedule entry {entry} declared no state '{name}'")
+        return self._named_states[(entry, name)]
 
     # --- what the engine uses ---------------------------------------------------------
     def acquire(self):

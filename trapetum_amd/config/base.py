@@ -130,7 +130,11 @@ def read_config_json(folder):
 
 
 def architecture_name(d):
+    """The model class a config.json names: the first entry of its 'architectures' list, or the string under
+    'architecture'."""
     archs = d.get("architectures")
-    if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError("config.json has no 'architectures' list naming the model class")
-    return archs[0]
+    if isinstance(archs, list) and archs and isinstance(archs[0], str):
+        return archs[0]
+    if isinstance(d.get("architecture"), str):
+        return d["architecture"]
+    raise ConfigError("config.json has no 'architectures' list (or 'architecture' string) naming the model class")

@@ -30,10 +30,14 @@ extern "C" int tp_embed_rows(const int* tokens, const void* table, int dtype, fl
 }
 
 // ---- RMSNorm: out = x * rsqrt(mean(x^2) + eps) * gain.  runtime/cuda/codebook_gemv.cu:192-202 ---------
+// A norm over `groups` equal consecutive parts of a row is the same norm over rows of the part's length, `groups`
+// times as many, part g of a row taking the g-th stretch of the gain: a block's row is blockIdx.x, its stretch
+// blockIdx.x % groups, and D is the part's length.
 template <typename TI, typename TO>
 __global__ void rms_norm_k(const TI* __restrict__ x, const float* __restrict__ gain, float eps,
-                           TO* __restrict__ out, int D) {
+                           TO* __restrict__ out, int D, int groups) {
     __shared__ float red[16];
+    gain += (size_t)(blockIdx.x % groups) * D;
     const TI* xr = x + (size_t)blockIdx.x * D;
     TO* orow = out + (size_t)blockIdx.x * D;
     float ss = 0.f;
@@ -46,8 +50,9 @@ __global__ void rms_norm_k(const TI* __restrict__ x, const float* __restrict__ g
 // the same for rows of at most 256 * EPT elements: every element is read once and kept in registers
 template <typename TI, typename TO, int EPT, int NTH>
 __global__ void __launch_bounds__(NTH)
-rms_norm_reg_k(const TI* __restrict__ x, const float* __restrict__ gain, float eps, TO* __restrict__ out, int D) {
+rms_norm_reg_k(const TI* __restrict__ x, const float* __restrict__ gain, float eps, TO* __restrict__ out, int D, int groups) {
     __shared__ float red[16];
+    gain += (size_t)(blockIdx.x % groups) * D;
     const TI* xr = x + (size_t)blockIdx.x * D;
     TO* orow = out + (size_t)blockIdx.x * D;
     float v[EPT], gn[EPT];
@@ -70,23 +75,25 @@ rms_norm_reg_k(const TI* __restrict__ x, const float* __restrict__ gain, float e
 }
 
 template <typename TI, typename TO>
-static void rms_norm_launch(const void* x, const float* gain, float eps, void* out, int M, int D, hipStream_t s) {
-    if (D <= 256 * 2) rms_norm_reg_k<TI, TO, 2, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
-    else if (M <= 128 && D <= 1024 * 4) rms_norm_reg_k<TI, TO, 4, 1024><<<M, 1024, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
-    else if (D <= 256 * 4) rms_norm_reg_k<TI, TO, 4, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
-    else if (D <= 256 * 12) rms_norm_reg_k<TI, TO, 12, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
-    else if (D <= 1024 * 8) rms_norm_reg_k<TI, TO, 8, 1024><<<M, 1024, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
-    else rms_norm_k<TI, TO><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+static void rms_norm_launch(const void* x, const float* gain, float eps, void* out, int M, int D, int groups, hipStream_t s) {
+    if (D <= 256 * 2) rms_norm_reg_k<TI, TO, 2, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D, groups);
+    else if (M <= 128 && D <= 1024 * 4) rms_norm_reg_k<TI, TO, 4, 1024><<<M, 1024, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D, groups);
+    else if (D <= 256 * 4) rms_norm_reg_k<TI, TO, 4, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D, groups);
+    else if (D <= 256 * 12) rms_norm_reg_k<TI, TO, 12, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D, groups);
+    else if (D <= 1024 * 8) rms_norm_reg_k<TI, TO, 8, 1024><<<M, 1024, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D, groups);
+    else rms_norm_k<TI, TO><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D, groups);
 }
 
 extern "C" int tp_rms_norm(const void* x, int in_dtype, const float* gain, float eps, void* out, int out_dtype,
-                           int M, int D, void* stream) {
+                           int M, int D, int groups, void* stream) {
     TP_REQUIRE(M > 0 && D > 0, "rms_norm: empty shape M=%d D=%d", M, D);
+    TP_REQUIRE(groups > 0 && D % groups == 0, "rms_norm: rows of %d elements cannot be cut into %d equal groups", D, groups);
+    M *= groups; D /= groups;
     hipStream_t s = (hipStream_t)stream;
-    if (in_dtype == TP_F32 && out_dtype == TP_F32) rms_norm_launch<float, float>(x, gain, eps, out, M, D, s);
-    else if (in_dtype == TP_F32 && out_dtype == TP_BF16) rms_norm_launch<float, bf16_t>(x, gain, eps, out, M, D, s);
-    else if (in_dtype == TP_BF16 && out_dtype == TP_F32) rms_norm_launch<bf16_t, float>(x, gain, eps, out, M, D, s);
-    else if (in_dtype == TP_BF16 && out_dtype == TP_BF16) rms_norm_launch<bf16_t, bf16_t>(x, gain, eps, out, M, D, s);
+    if (in_dtype == TP_F32 && out_dtype == TP_F32) rms_norm_launch<float, float>(x, gain, eps, out, M, D, groups, s);
+    else if (in_dtype == TP_F32 && out_dtype == TP_BF16) rms_norm_launch<float, bf16_t>(x, gain, eps, out, M, D, groups, s);
+    else if (in_dtype == TP_BF16 && out_dtype == TP_F32) rms_norm_launch<bf16_t, float>(x, gain, eps, out, M, D, groups, s);
+    else if (in_dtype == TP_BF16 && out_dtype == TP_BF16) rms_norm_launch<bf16_t, bf16_t>(x, gain, eps, out, M, D, groups, s);
     else return tp_fail("rms_norm: unknown dtypes %d -> %d", in_dtype, out_dtype);
     return tp_check_launch("rms_norm");
 }
@@ -97,8 +104,10 @@ template <typename T>
 __global__ void add_rms_norm_k(float* __restrict__ stream, const T* __restrict__ rows,
                                const float* __restrict__ gain_post, float eps_post,
                                const float* __restrict__ gain_next, float eps_next,
-                               T* __restrict__ out, int D) {
+                               T* __restrict__ out, int D, int groups) {
     __shared__ float red[16];
+    if (gain_post) gain_post += (size_t)(blockIdx.x % groups) * D;
+    if (gain_next) gain_next += (size_t)(blockIdx.x % groups) * D;
     float* sr = stream + (size_t)blockIdx.x * D;
     const T* ar = rows + (size_t)blockIdx.x * D;
     float scale_a = 1.f;
@@ -129,8 +138,10 @@ template <typename TR, typename T, int EPT, int NTH>
 __global__ void __launch_bounds__(NTH)
 add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int n_slices, long slice_stride,
                    const float* __restrict__ gain_post, float eps_post,
-                   const float* __restrict__ gain_next, float eps_next, T* __restrict__ out, int D) {
+                   const float* __restrict__ gain_next, float eps_next, T* __restrict__ out, int D, int groups) {
     __shared__ float red[16];
+    if (gain_post) gain_post += (size_t)(blockIdx.x % groups) * D;
+    if (gain_next) gain_next += (size_t)(blockIdx.x % groups) * D;
     float* sr = stream + (size_t)blockIdx.x * D;
     const TR* ar = rows + (size_t)blockIdx.x * D;
     float a[EPT], v[EPT], gp[EPT], gn[EPT];
@@ -210,8 +221,10 @@ template <typename TR, typename T, int CPT, int NTH>
 __global__ void __launch_bounds__(NTH)
 add_rms_norm_vec_k(float* __restrict__ stream, const TR* __restrict__ rows, int n_slices, long slice_stride,
                    const float* __restrict__ gain_post, float eps_post,
-                   const float* __restrict__ gain_next, float eps_next, T* __restrict__ out, int D) {
+                   const float* __restrict__ gain_next, float eps_next, T* __restrict__ out, int D, int groups) {
     __shared__ float red[16], red_next[16];             // one for each of the two sums: no barrier between their uses
+    if (gain_post) gain_post += (size_t)(blockIdx.x % groups) * D;
+    if (gain_next) gain_next += (size_t)(blockIdx.x % groups) * D;
     float* sr = stream + (size_t)blockIdx.x * D;
     const TR* ar = rows + (size_t)blockIdx.x * D;
     float a[CPT][4], v[CPT][4], gp[CPT][4], gn[CPT][4];
@@ -287,7 +300,7 @@ add_rms_norm_vec_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
 
 template <typename TR, typename T>
 static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, long slice_stride, const float* gp, float ep,
-                               const float* gn, float en, void* out, int M, int D, hipStream_t s) {
+                               const float* gn, float en, void* out, int M, int D, int groups, hipStream_t s) {
     // few rows: many threads per row (the kernel is bound by the latency of its loads, not by their volume)
     // few rows: a chunk a lane and as many lanes as the row has chunks (the kernel is bound by the latency of its loads:
     // one 16-byte load per operand and lane; 2B decode of 64 sequences 3.51 -> 3.21 ms a step against 1,024 lanes of
@@ -296,7 +309,7 @@ static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, lo
                          (!gp || (uintptr_t)gp % 16 == 0) && (!gn || (uintptr_t)gn % 16 == 0) && (!out || (uintptr_t)out % 16 == 0);
     const bool few = aligned && M <= 128, vec = aligned && M > 128;
     // (HipOps.add_rms_norm adds the slices itself, with sum_slices, before it comes here with a wider row)
-#define TP_ADD_NORM_VEC(CPT, NTH) add_rms_norm_vec_k<TR, T, CPT, NTH><<<M, NTH, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D)
+#define TP_ADD_NORM_VEC(CPT, NTH) add_rms_norm_vec_k<TR, T, CPT, NTH><<<M, NTH, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D, groups)
     if (few && D > 256 * 4 && D <= 640 * 4) TP_ADD_NORM_VEC(1, 640);
     else if (few && D > 640 * 4 && D <= 1024 * 4) TP_ADD_NORM_VEC(1, 1024);
     else if (few && D > 1024 * 4 && D <= 640 * 8) TP_ADD_NORM_VEC(2, 640);
@@ -313,12 +326,12 @@ static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, lo
     else if (vec && D <= 448 * 12) TP_ADD_NORM_VEC(3, 448);
     else if (vec && D <= 512 * 12) TP_ADD_NORM_VEC(3, 512);
     else if (vec && D <= 512 * 16) TP_ADD_NORM_VEC(4, 512);
-    else if (D <= 256 * 2) add_rms_norm_reg_k<TR, T, 2, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
-    else if (M <= 128 && D <= 1024 * 4) add_rms_norm_reg_k<TR, T, 4, 1024><<<M, 1024, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
-    else if (D <= 256 * 4) add_rms_norm_reg_k<TR, T, 4, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
-    else if (D <= 256 * 12) add_rms_norm_reg_k<TR, T, 12, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
-    else if (D <= 1024 * 8) add_rms_norm_reg_k<TR, T, 8, 1024><<<M, 1024, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
-    else if (n_slices == 1 && sizeof(TR) == sizeof(T)) add_rms_norm_k<T><<<M, 256, 0, s>>>(stream, (const T*)rows, gp, ep, gn, en, (T*)out, D);
+    else if (D <= 256 * 2) add_rms_norm_reg_k<TR, T, 2, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D, groups);
+    else if (M <= 128 && D <= 1024 * 4) add_rms_norm_reg_k<TR, T, 4, 1024><<<M, 1024, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D, groups);
+    else if (D <= 256 * 4) add_rms_norm_reg_k<TR, T, 4, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D, groups);
+    else if (D <= 256 * 12) add_rms_norm_reg_k<TR, T, 12, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D, groups);
+    else if (D <= 1024 * 8) add_rms_norm_reg_k<TR, T, 8, 1024><<<M, 1024, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D, groups);
+    else if (n_slices == 1 && sizeof(TR) == sizeof(T)) add_rms_norm_k<T><<<M, 256, 0, s>>>(stream, (const T*)rows, gp, ep, gn, en, (T*)out, D, groups);
     else return tp_fail("add_rms_norm: rows in slices need a width of at most %d, found %d", 1024 * 8, D);
 #undef TP_ADD_NORM_VEC
     return 0;
@@ -326,15 +339,17 @@ static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, lo
 
 extern "C" int tp_add_rms_norm(float* stream, const void* rows, int rows_dtype, int n_slices, long slice_stride,
                                const float* gain_post, float eps_post, const float* gain_next, float eps_next,
-                               void* out, int out_dtype, int M, int D, void* stream_) {
+                               void* out, int out_dtype, int M, int D, int groups, void* stream_) {
     TP_REQUIRE(M > 0 && D > 0, "add_rms_norm: empty shape M=%d D=%d", M, D);
+    TP_REQUIRE(groups > 0 && D % groups == 0, "add_rms_norm: rows of %d elements cannot be cut into %d equal groups", D, groups);
+    M *= groups; D /= groups;                        // see rms_norm_k
     TP_REQUIRE(!gain_next || out, "add_rms_norm: a next norm needs an output buffer");
     TP_REQUIRE(n_slices >= 1 && (n_slices == 1 || rows_dtype == TP_F32), "add_rms_norm: rows in %d slices must be float32", n_slices);
     hipStream_t s = (hipStream_t)stream_;
     int rc;
-    if (rows_dtype == TP_BF16 && out_dtype == TP_BF16) rc = add_rms_norm_launch<bf16_t, bf16_t>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, s);
-    else if (rows_dtype == TP_F32 && out_dtype == TP_F32) rc = add_rms_norm_launch<float, float>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, s);
-    else if (rows_dtype == TP_F32 && out_dtype == TP_BF16) rc = add_rms_norm_launch<float, bf16_t>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, s);
+    if (rows_dtype == TP_BF16 && out_dtype == TP_BF16) rc = add_rms_norm_launch<bf16_t, bf16_t>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, groups, s);
+    else if (rows_dtype == TP_F32 && out_dtype == TP_F32) rc = add_rms_norm_launch<float, float>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, groups, s);
+    else if (rows_dtype == TP_F32 && out_dtype == TP_BF16) rc = add_rms_norm_launch<float, bf16_t>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, groups, s);
     else return tp_fail("add_rms_norm: unsupported dtypes rows %d -> out %d", rows_dtype, out_dtype);
     if (rc) return rc;
     return tp_check_launch("add_rms_norm");
@@ -631,6 +646,19 @@ extern "C" int tp_add_bias(void* rows, int dtype, const float* bias, int M, int 
     else if (dtype == TP_F32) add_bias_k<float><<<(unsigned)blocks, 256, 0, s>>>((float*)rows, bias, total, N);
     else return tp_fail("add_bias: unknown dtype %d", dtype);
     return tp_check_launch("add_bias");
+}
+
+// ---- rows *= scale (float32, in place): logits that a model multiplies by a constant ------------------------------
+__global__ void scale_rows_k(float* __restrict__ x, long total, float scale) {
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) x[i] *= scale;
+}
+
+extern "C" int tp_scale_rows(float* x, long total, float scale, void* stream) {
+    TP_REQUIRE(x && total > 0, "scale_rows: empty operand");
+    long blocks = (total + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    scale_rows_k<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(x, total, scale);
+    return tp_check_launch("scale_rows");
 }
 
 template <typename T>

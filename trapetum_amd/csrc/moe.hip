@@ -1,0 +1,188 @@
+// A mixture of experts: the router's choice, the step's (token, expert) pairs sorted by expert, the experts' two
+// products over runs of pairs, and the weighted sum per token.  Nothing here returns to the host: the number of pairs
+// an expert gets lives on the device, and launches are sized for the worst case.
+#include "common.h"
+#include "tile.h"
+
+// ---- scores = softmax(logits) over all experts; the `top` largest (ties: the smaller index) and their scores --------
+// grid (rows), one wave a row; dynamic LDS: E floats
+__global__ void __launch_bounds__(64)
+route_top_k(const float* __restrict__ logits, int E, int top, int renormalize, int* __restrict__ chosen, float* __restrict__ weight) {
+    extern __shared__ float sc[];
+    const int r = blockIdx.x, lane = threadIdx.x;
+    const float* z = logits + (size_t)r * E;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) { const float p = expf(z[e] - mx); sc[e] = p; sum += p; }
+    sum = wave_sum(sum);
+    __syncthreads();
+    float kept = 0.f;
+    for (int k = 0; k < top; k++) {
+        float best = -1.f;
+        int at = E;
+        for (int e = lane; e < E; e += 64) if (sc[e] > best) { best = sc[e]; at = e; }     // ascending e: the first of equals stays
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, 64);
+            const int oa = __shfl_xor(at, o, 64);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+        }
+        if (lane == 0) {
+            chosen[(size_t)r * top + k] = at;
+            weight[(size_t)r * top + k] = best / sum;
+            sc[at] = -1.f;                               // scores are positive: a chosen expert is not chosen again
+        }
+        kept += best / sum;
+        __syncthreads();
+    }
+    if (renormalize && lane == 0)
+        for (int k = 0; k < top; k++) weight[(size_t)r * top + k] /= kept;
+}
+
+extern "C" int tp_route_top(const float* logits, int M, int E, int top, int renormalize, int* chosen, float* weight, void* stream) {
+    TP_REQUIRE(M > 0 && E > 0 && top > 0 && top <= E, "route_top: %d of %d experts for %d rows", top, E, M);
+    TP_REQUIRE(logits && chosen && weight, "route_top: a null operand");
+    TP_REQUIRE((size_t)E * sizeof(float) <= 60000, "route_top: %d experts exceed the kernel's table", E);
+    route_top_k<<<M, 64, (size_t)E * sizeof(float), (hipStream_t)stream>>>(logits, E, top, renormalize, chosen, weight);
+    return tp_check_launch("route_top");
+}
+
+// ---- pairs sorted by expert: order[i] = the pair at sorted place i, place[pair] = its sorted place, first[e] = where
+// expert e's run starts (first[E] = P).  Pairs of one expert keep their order.  grid (experts), 256 threads ---------
+__global__ void __launch_bounds__(256)
+expert_sort_k(const int* __restrict__ chosen, int P, int E, int* __restrict__ order, int* __restrict__ place, int* __restrict__ first) {
+    __shared__ int wave_n[4];
+    __shared__ int below_s[4];
+    const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int below = 0;
+    for (int p = tid; p < P; p += 256) below += chosen[p] < e ? 1 : 0;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) below += __shfl_xor(below, o, 64);
+    if (lane == 0) below_s[wave] = below;
+    __syncthreads();
+    const int start = below_s[0] + below_s[1] + below_s[2] + below_s[3];
+    int base = start;
+    for (int p0 = 0; p0 < P; p0 += 256) {
+        const int p = p0 + tid;
+        const bool mine = p < P && chosen[p] == e;
+        const unsigned long long mask = __ballot(mine);
+        if (lane == 0) wave_n[wave] = __popcll(mask);
+        __syncthreads();
+        int before = __popcll(mask & ((1ull << lane) - 1ull));
+        for (int w = 0; w < wave; w++) before += wave_n[w];
+        if (mine) { order[base + before] = p; place[p] = base + before; }
+        base += wave_n[0] + wave_n[1] + wave_n[2] + wave_n[3];
+        __syncthreads();
+    }
+    if (tid == 0) {
+        first[e] = start;
+        if (e == E - 1) first[E] = P;
+    }
+}
+
+// ---- an expert's products over its run of pairs.  Tiles of TM pairs of one expert x TN columns; grid (column tiles,
+// row tiles for the worst case): a block finds its expert and tile by walking first[], one past the end leaves.
+// GATED: rows of X gathered by pair (token = pair / top), W [E, 2 F, K] (gate rows, then up rows),
+//        y = min(g, limit) * sigmoid(alpha min(g, limit)) * (clamp(u, -limit, limit) + shift)  -> T [P, F] by sorted place;
+// else:  rows of A = sorted places themselves, W [E, N, K], out float [P, N] by sorted place.
+template <typename T, bool GATED, int TM>
+__global__ void __launch_bounds__(256)
+expert_linear_k(const T* __restrict__ a, const T* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
+                int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out) {
+    constexpr int TN = 64, BK = 16;
+    __shared__ TileShared<TM, GATED ? 2 * TN : TN, BK> sh;
+    int t = blockIdx.y, e = 0, lo = 0, hi = 0;
+    for (; e < E; e++) {
+        lo = first[e]; hi = first[e + 1];
+        const int tiles = (hi - lo + TM - 1) / TM;
+        if (t < tiles) break;
+        t -= tiles;
+    }
+    if (e == E) return;
+    const int p0 = lo + t * TM, n0 = blockIdx.x * TN;
+    const T* we = w + (size_t)e * (GATED ? 2 : 1) * N * K;
+    const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+    if constexpr (GATED) {
+        float acc[TM / 16][2 * TN / 16];                 // columns 0 .. TN - 1: gate, TN .. 2 TN - 1: up, of the same units
+        tile_product<TM, 2 * TN, BK>(acc, K,
+            [&](int m, int k) { return p0 + m < hi ? ld_f32(a + (size_t)(order[p0 + m] / top) * K + k) : 0.f; },
+            [&](int n, int k) { const int u = n0 + (n & (TN - 1)); return u < N ? ld_f32(we + ((size_t)(n >= TN ? N : 0) + u) * K + k) : 0.f; }, sh);
+#pragma unroll
+        for (int i = 0; i < TM / 16; i++)
+#pragma unroll
+            for (int j = 0; j < TN / 16; j++) {
+                const int p = p0 + ty + 16 * i, n = n0 + tx + 16 * j;
+                if (p >= hi || n >= N) continue;
+                const float g = fminf(acc[i][j], limit), u = fminf(fmaxf(acc[i][j + TN / 16], -limit), limit);
+                st_f32((T*)out + (size_t)p * N + n, g / (1.f + expf(-alpha * g)) * (u + shift));
+            }
+    } else {
+        float acc[TM / 16][TN / 16];
+        tile_product<TM, TN, BK>(acc, K,
+            [&](int m, int k) { return p0 + m < hi ? ld_f32(a + (size_t)(p0 + m) * K + k) : 0.f; },
+            [&](int n, int k) { return n0 + n < N ? ld_f32(we + (size_t)(n0 + n) * K + k) : 0.f; }, sh);
+#pragma unroll
+        for (int i = 0; i < TM / 16; i++)
+#pragma unroll
+            for (int j = 0; j < TN / 16; j++) {
+                const int p = p0 + ty + 16 * i, n = n0 + tx + 16 * j;
+                if (p < hi && n < N) ((float*)out)[(size_t)p * N + n] = acc[i][j];
+            }
+    }
+}
+
+// ---- out[m] = sum_k weight[m, k] * pair_out[place[m top + k]], k ascending, float32.  grid (rows, column blocks) ------
+__global__ void __launch_bounds__(256)
+expert_combine_k(const float* __restrict__ pair_out, const int* __restrict__ place, const float* __restrict__ weight, int top, int D,
+                 float* __restrict__ out) {
+    const int m = blockIdx.x, d = blockIdx.y * 256 + threadIdx.x;
+    if (d >= D) return;
+    float acc = 0.f;
+    for (int k = 0; k < top; k++)
+        acc = __builtin_fmaf(weight[(size_t)m * top + k], pair_out[(size_t)place[(size_t)m * top + k] * D + d], acc);
+    out[(size_t)m * D + d] = acc;
+}
+
+// workspace: order [P], place [P], first [E + 1] (int32), then y [P, F] of the activation dtype, then pair_out [P, D] float
+static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+extern "C" long tp_expert_ffn_workspace_bytes(int dtype, int M, int top, int E, int F, int D) {
+    const size_t P = (size_t)M * top, el = dtype == TP_BF16 ? 2 : 4;
+    return (long)(align256((2 * P + E + 1) * sizeof(int)) + align256(P * F * el) + align256(P * D * sizeof(float)));
+}
+
+extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* chosen, const float* weight, int top, int E, int F,
+                             const void* w_gate_up, const void* w_down, float limit, float alpha, float shift,
+                             void* workspace, long workspace_bytes, float* out, void* stream) {
+    TP_REQUIRE(M > 0 && D > 0 && top > 0 && E > 0 && F > 0, "expert_ffn: empty shape M=%d D=%d top=%d E=%d F=%d", M, D, top, E, F);
+    TP_REQUIRE(x && chosen && weight && w_gate_up && w_down && workspace && out, "expert_ffn: a null operand");
+    TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F32, "expert_ffn: unknown dtype %d", dtype);
+    TP_REQUIRE(workspace_bytes >= tp_expert_ffn_workspace_bytes(dtype, M, top, E, F, D), "expert_ffn: a workspace of %ld bytes is too small", workspace_bytes);
+    TP_REQUIRE(E <= 65535 && (long)M * top < (1L << 30), "expert_ffn: too many experts or pairs for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    const int P = M * top;
+    const size_t el = dtype == TP_BF16 ? 2 : 4;
+    int* order = (int*)workspace;
+    int* place = order + P;
+    int* first = place + P;
+    char* y = (char*)workspace + align256((2 * (size_t)P + E + 1) * sizeof(int));
+    float* pair_out = (float*)(y + align256((size_t)P * F * el));
+    expert_sort_k<<<E, 256, 0, s>>>(chosen, P, E, order, place, first);
+    if (int rc = tp_check_launch("expert_ffn (sort)")) return rc;
+    const bool few = P <= 64;                            // a decode step: most runs hold a pair or two
+    const int TM = few ? 16 : 64;
+    const int row_tiles = tp_cdiv(P, TM) + (E < P ? E : P);
+    TP_REQUIRE(row_tiles <= 65535, "expert_ffn: %d row tiles exceed one launch", row_tiles);
+#define TP_EXPERT(T, G, TMv, Nv, Kv, A, W, O) expert_linear_k<T, G, TMv><<<dim3(tp_cdiv(Nv, 64), row_tiles), 256, 0, s>>>( \
+        (const T*)(A), (const T*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O)
+    if (dtype == TP_BF16) { if (few) TP_EXPERT(bf16_t, true, 16, F, D, x, w_gate_up, y); else TP_EXPERT(bf16_t, true, 64, F, D, x, w_gate_up, y); }
+    else { if (few) TP_EXPERT(float, true, 16, F, D, x, w_gate_up, y); else TP_EXPERT(float, true, 64, F, D, x, w_gate_up, y); }
+    if (int rc = tp_check_launch("expert_ffn (gate, up)")) return rc;
+    if (dtype == TP_BF16) { if (few) TP_EXPERT(bf16_t, false, 16, D, F, y, w_down, pair_out); else TP_EXPERT(bf16_t, false, 64, D, F, y, w_down, pair_out); }
+    else { if (few) TP_EXPERT(float, false, 16, D, F, y, w_down, pair_out); else TP_EXPERT(float, false, 64, D, F, y, w_down, pair_out); }
+#undef TP_EXPERT
+    if (int rc = tp_check_launch("expert_ffn (down)")) return rc;
+    expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, place, weight, top, D, out);
+    return tp_check_launch("expert_ffn (combine)");
+}

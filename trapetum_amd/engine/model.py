@@ -18,16 +18,20 @@ from .batch import StepContext, StepError, classify
 class AssembledLayer:
     def __init__(self, lspec):
         mixer = build_part("mixer", lspec.mixer)
-        ff = build_part("feed_forward", lspec.feed_forward)
+        ff = build_part("feed_forward", lspec.feed_forward) if lspec.feed_forward is not None else None
         block_cls = part_class("block", lspec.block[0])
         unknown = set(lspec.norms or {}) - set(block_cls.norm_sites())
         if unknown:
             raise ValueError(f"the layer's spec names norms for {sorted(unknown)}, block '{lspec.block[0]}' has {list(block_cls.norm_sites())}")
         self.block = block_cls(mixer, ff, lambda site: build_part("norm", lspec.norm_of(site)), **lspec.block[1])
         self.prefixes = lspec.prefixes
-        self.places = [(mixer, self._prefix("mixer")), (ff, self._prefix("feed_forward"))]
+        self.places = [(mixer, self._prefix("mixer"))]
+        if ff is not None:
+            self.places.append((ff, self._prefix("feed_forward")))
         for site, norm in self.block.norms.items():
             self.places.append((norm, self._prefix(site)))
+        for site, part in self.block.inner_parts().items():
+            self.places.append((part, self._prefix(site)))
         if self.block.tensor_specs():
             self.places.append((self.block, self._prefix("block")))
 
@@ -88,11 +92,15 @@ class Model:
             specs.append(None if e.cache_of is not None else self.layers[e.layer].block.mixer.cache_spec())
         return specs
 
+    def entry_state_specs(self):
+        """For every schedule entry the states its block keeps beside the mixer's cache, by name."""
+        return [self.layers[e.layer].block.state_specs() for e in self.schedule]
+
     def new_cache(self, max_tokens, max_context=None, max_slots=None, page_size=64):
         max_context = max_context or max_tokens
         max_slots = max_slots or max(1, -(-max_tokens // page_size))
         return ModelCache(self.entry_cache_specs(), max_tokens, max_context, max_slots, page_size,
-                          self.rt.dtype, self.rt.device)
+                          self.rt.dtype, self.rt.device, entry_states=self.entry_state_specs())
 
     # --- the step -----------------------------------------------------------------------
     def step(self, cache, slots, tokens, counts=None, want=None):

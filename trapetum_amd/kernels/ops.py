@@ -15,8 +15,15 @@ _P, _I, _L, _F = _c.c_void_p, _c.c_int, _c.c_long, _c.c_float
 
 _CORE_SIGS = {
     "tp_embed_rows": [_P, _P, _I, _F, _P, _I, _I, _I, _P],
-    "tp_rms_norm": [_P, _I, _P, _F, _P, _I, _I, _I, _P],
-    "tp_add_rms_norm": [_P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _I, _I, _I, _P],
+    "tp_rms_norm": [_P, _I, _P, _F, _P, _I, _I, _I, _I, _P],
+    "tp_add_rms_norm": [_P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _I, _I, _I, _I, _P],
+    "tp_scale_rows": [_P, _L, _F, _P],
+    "tp_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "tp_latent_prepare": [_P, _L, _I, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _P],
+    "tp_head_linear": [_P, _L, _L, _P, _P, _L, _L, _I, _I, _I, _I, _I, _P],
+    "tp_route_top": [_P, _I, _I, _I, _I, _P, _P, _P],
+    "tp_expert_ffn_workspace_bytes": [_I, _I, _I, _I, _I, _I],
+    "tp_expert_ffn": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _P, _F, _F, _F, _P, _L, _P, _P],
     "tp_gather_rows": [_P, _P, _P, _I, _I, _I, _P],
     "tp_sum_slices": [_P, _I, _L, _P, _I, _L, _P],
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
@@ -193,7 +200,8 @@ class HipOps:
                    out.data_ptr(), m, d, v, self._stream())
         return out
 
-    def rms_norm(self, x, gain, eps, out_dtype):
+    def rms_norm(self, x, gain, eps, out_dtype, groups=1):
+        """groups: the row is cut into that many equal consecutive parts, each over its own root mean square."""
         self._dev(x, gain)
         if not x.is_contiguous() or x.dim() != 2:
             raise KernelError("rms_norm: rows must be a contiguous matrix")
@@ -201,13 +209,18 @@ class HipOps:
         if gain.dtype != torch.float32 or gain.numel() != d or not gain.is_contiguous():
             raise KernelError(f"rms_norm: gain must be float32 [{d}]")
         out = torch.empty((m, d), dtype=out_dtype, device=self.device)
+        if groups < 1 or d % groups:
+            raise KernelError(f"rms_norm: rows of {d} elements cannot be cut into {groups} equal groups")
         self._call(self.lib, "tp_rms_norm", x.data_ptr(), _code(x.dtype), gain.data_ptr(), float(eps), out.data_ptr(),
-                   _code(out_dtype), m, d, self._stream())
+                   _code(out_dtype), m, d, int(groups), self._stream())
         return out
 
-    def add_rms_norm(self, stream, rows, gain_post, eps_post, gain_next, eps_next, out_dtype):
-        """stream += post-norm(rows) (or rows); returns next-norm(stream) or None.  rows: a tensor or SplitRows."""
+    def add_rms_norm(self, stream, rows, gain_post, eps_post, gain_next, eps_next, out_dtype, groups=1):
+        """stream += post-norm(rows) (or rows); returns next-norm(stream) or None.  rows: a tensor or SplitRows.
+        groups: both norms cut the row into that many equal consecutive parts."""
         m, d = stream.shape
+        if groups < 1 or d % groups:
+            raise KernelError(f"add_rms_norm: rows of {d} elements cannot be cut into {groups} equal groups")
         n_slices, stride = 1, 0
         if isinstance(rows, SplitRows) and d > self.MAX_SLICED_WIDTH:
             rows = self.rows(rows, out_dtype)            # the fused kernel keeps a row in registers: wider rows are added first
@@ -226,7 +239,131 @@ class HipOps:
         self._call(self.lib, "tp_add_rms_norm", stream.data_ptr(), rows.data_ptr(), _code(rows.dtype), n_slices, stride,
                    gain_post.data_ptr() if gain_post is not None else None, float(eps_post),
                    gain_next.data_ptr() if gain_next is not None else None, float(eps_next),
-                   out.data_ptr() if out is not None else None, _code(out_dtype), m, d, self._stream())
+                   out.data_ptr() if out is not None else None, _code(out_dtype), m, d, int(groups), self._stream())
+        return out
+
+    def scale_rows(self, x, scale):
+        """x *= scale, in place (float32)."""
+        self._dev(x)
+        if x.dtype != torch.float32 or not x.is_contiguous():
+            raise KernelError("scale_rows: expected a contiguous float32 tensor")
+        self._call(self.lib, "tp_scale_rows", x.data_ptr(), x.numel(), float(scale), self._stream())
+
+    def causal_conv(self, stream, w, state, slot_ids, cu_rows, row_seq, out_dtype, residual=True, one_row_each=False):
+        """out[r] = (stream[r]) + sum_j w[:, j] * stream[r - (taps - 1) + j] within each sequence; the rows before the
+        step are read from state[slot] (float32 [slots, taps - 1, D], oldest first), which then takes the last
+        taps - 1 rows of (state, step).  one_row_each: every sequence brings one row (one launch does both)."""
+        self._dev(stream, w, state, slot_ids, cu_rows, row_seq)
+        if stream.dtype != torch.float32 or stream.dim() != 2 or not stream.is_contiguous():
+            raise KernelError("causal_conv: the stream must be contiguous float32 [rows, channels]")
+        m, d = stream.shape
+        if w.dtype != torch.float32 or w.dim() != 2 or w.shape[0] != d or not w.is_contiguous():
+            raise KernelError(f"causal_conv: the taps must be contiguous float32 [{d}, taps]")
+        taps, n_seq = w.shape[1], cu_rows.numel() - 1
+        for t, n in ((cu_rows, n_seq + 1), (row_seq, m), (slot_ids, n_seq)):
+            if t.dtype != torch.int32 or t.numel() != n:
+                raise KernelError("causal_conv: cu_rows, row_seq and slot_ids must be int32 of the step's geometry")
+        if taps > 1 and (state is None or state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (taps - 1, d)
+                         or not state.is_contiguous()):
+            raise KernelError(f"causal_conv: the state must be contiguous float32 [slots, {taps - 1}, {d}]")
+        out = torch.empty((m, d), dtype=out_dtype, device=self.device)
+        self._call(self.lib, "tp_causal_conv", stream.data_ptr(), w.data_ptr(), state.data_ptr() if taps > 1 else None,
+                   slot_ids.data_ptr(), cu_rows.data_ptr(), row_seq.data_ptr(), out.data_ptr(), _code(out_dtype), m, n_seq, d, taps,
+                   1 if residual else 0, 1 if one_row_each else 0, self._stream())
+        return out
+
+    # ---- attention through a cached latent ---------------------------------------------------------------------
+    def latent_prepare(self, proj, H, dn, dr, R, gain, eps, inv_freq, rot, row_seq, row_pos, new_len, table, pool, rows_cap,
+                       own=True, out_dtype=None):
+        """proj [M, H (dr + dn) (+ dr + R)]: per head [rotated | unrotated] query parts, then (own) [key part | latent].
+        Returns q [M, H (dr + R)] with every head's first dr elements set (the rotated query part; the rest is left
+        for `head_linear`) and, when own, the step's rows [rope(key part) | rmsnorm(latent) * gain] [M, dr + R], which
+        are also written into the cache pool [pages, 1, page, dr + R]."""
+        self._dev(proj, gain, inv_freq, row_seq, row_pos, new_len, table, pool)
+        m = proj.shape[0]
+        stride = self._rows(proj, "latent_prepare proj")
+        width = H * (dr + dn) + ((dr + R) if own else 0)
+        if proj.shape[1] != width or (out_dtype is not None and out_dtype != proj.dtype):
+            raise KernelError(f"latent_prepare: rows of {proj.shape[1]} columns, this geometry needs {width} of the output's dtype")
+        if rot and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rot // 2):
+            raise KernelError(f"latent_prepare: a rotation over {rot} needs float32 inv_freq [{rot // 2}]")
+        for t in (row_seq, row_pos):
+            if t.dtype != torch.int32 or t.numel() != m:
+                raise KernelError("latent_prepare: row_seq and row_pos must be int32, one entry per row")
+        q = torch.empty((m, H * (dr + R)), dtype=proj.dtype, device=self.device)
+        mine = None
+        page = table_w = 1
+        if own:
+            if gain is None or gain.dtype != torch.float32 or gain.numel() != R or not gain.is_contiguous():
+                raise KernelError(f"latent_prepare: the latent's gain must be contiguous float32 [{R}]")
+            self._check_pools("latent_prepare", proj.dtype, new_len.numel(), 1, dr + R, new_len, table, pool, pool)
+            page, table_w = pool.shape[2], table.shape[1]
+            mine = torch.empty((m, dr + R), dtype=proj.dtype, device=self.device)
+        self._call(self.lib, "tp_latent_prepare", proj.data_ptr(), stride, _code(proj.dtype), m, H, dn, dr, R,
+                   gain.data_ptr() if own else None, float(eps), inv_freq.data_ptr() if rot else None, int(rot),
+                   row_seq.data_ptr(), row_pos.data_ptr(), new_len.data_ptr(), table.data_ptr() if own else None, table_w,
+                   pool.data_ptr() if own else None, page, rows_cap if own else 0, q.data_ptr(),
+                   mine.data_ptr() if own else None, 1 if own else 0, self._stream())
+        return q, mine
+
+    def head_linear(self, x, w, out=None):
+        """out[m, h, :] = w[h] @ x[m, h, :].  x: a view [M, H, K] of wider rows (a head's elements contiguous), w
+        contiguous [H, N, K]; out: a view [M, H, N] to fill, or None for a new contiguous tensor."""
+        self._dev(x, w, out)
+        if x.dim() != 3 or w.dim() != 3 or w.shape[0] != x.shape[1] or w.shape[2] != x.shape[2] or not w.is_contiguous() or x.dtype != w.dtype:
+            raise KernelError(f"head_linear: rows {tuple(x.shape)} and matrices {tuple(w.shape)} do not fit, or differ in dtype")
+        m, H, K = x.shape
+        N = w.shape[1]
+        if out is None:
+            out = torch.empty((m, H, N), dtype=x.dtype, device=self.device)
+        if out.dim() != 3 or tuple(out.shape) != (m, H, N) or out.dtype != x.dtype:
+            raise KernelError(f"head_linear: the output must be {(m, H, N)} of {x.dtype}")
+        for t, what in ((x, "rows"), (out, "output")):
+            if t.shape[2] > 1 and t.stride(2) != 1:
+                raise KernelError(f"head_linear: a head's elements must be contiguous in the {what}")
+        self._call(self.lib, "tp_head_linear", x.data_ptr(), x.stride(0), x.stride(1), w.data_ptr(), out.data_ptr(),
+                   out.stride(0), out.stride(1), _code(x.dtype), m, H, N, K, self._stream())
+        return out
+
+    # ---- mixture of experts ------------------------------------------------------------------------------------
+    def route_top(self, logits, top, renormalize=False):
+        """softmax over all experts; the `top` largest scores (ties: the smaller index): int32 [M, top], float32 [M, top]."""
+        self._dev(logits)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
+            raise KernelError("route_top: router logits must be contiguous float32 [rows, experts]")
+        m, e = logits.shape
+        if not 0 < top <= e:
+            raise KernelError(f"route_top: {top} of {e} experts cannot be chosen")
+        chosen = torch.empty((m, top), dtype=torch.int32, device=self.device)
+        weight = torch.empty((m, top), dtype=torch.float32, device=self.device)
+        self._call(self.lib, "tp_route_top", logits.data_ptr(), m, e, int(top), 1 if renormalize else 0, chosen.data_ptr(),
+                   weight.data_ptr(), self._stream())
+        return chosen, weight
+
+    def expert_ffn(self, x, chosen, weights, w_gate_up, w_down, limit, alpha, shift):
+        """float32 [M, D]: sum over a row's chosen experts of weight * W_down,e (g' sigmoid(alpha g') (u' + shift)), with
+        g' = min(W_gate,e x, limit), u' = clamp(W_up,e x, -limit, limit).  w_gate_up [E, 2 F, D] (gate rows, then up
+        rows), w_down [E, D, F]."""
+        self._dev(x, chosen, weights, w_gate_up, w_down)
+        if x.dim() != 2 or not x.is_contiguous() or x.dtype != w_gate_up.dtype or x.dtype != w_down.dtype:
+            raise KernelError("expert_ffn: rows and matrices must be contiguous and of one dtype")
+        m, d = x.shape
+        if w_gate_up.dim() != 3 or w_down.dim() != 3 or not w_gate_up.is_contiguous() or not w_down.is_contiguous():
+            raise KernelError("expert_ffn: the experts' matrices must be contiguous [experts, rows, columns]")
+        e, f2, _ = w_gate_up.shape
+        f = f2 // 2
+        if f2 % 2 or w_gate_up.shape[2] != d or tuple(w_down.shape) != (e, d, f):
+            raise KernelError(f"expert_ffn: matrices {tuple(w_gate_up.shape)} and {tuple(w_down.shape)} do not fit rows of {d}")
+        top = chosen.shape[1]
+        if chosen.dtype != torch.int32 or tuple(chosen.shape) != (m, top) or weights.dtype != torch.float32 or tuple(weights.shape) != (m, top) \
+                or not chosen.is_contiguous() or not weights.is_contiguous():
+            raise KernelError("expert_ffn: the choice must be int32 [rows, top] with float32 weights of the same shape")
+        nbytes = self.lib.tp_expert_ffn_workspace_bytes(_code(x.dtype), m, top, e, f, d)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        out = torch.empty((m, d), dtype=torch.float32, device=self.device)
+        self._call(self.lib, "tp_expert_ffn", x.data_ptr(), _code(x.dtype), m, d, chosen.data_ptr(), weights.data_ptr(), top, e, f,
+                   w_gate_up.data_ptr(), w_down.data_ptr(), float(limit), float(alpha), float(shift), ws.data_ptr(), nbytes,
+                   out.data_ptr(), self._stream())
         return out
 
     MAX_SLICED_WIDTH = 8192        # widest row `add_rms_norm` takes in K slices

@@ -15,7 +15,7 @@ PartRef = Tuple[str, dict]          # (registered name, constructor parameters)
 class TensorSpec:
     """One tensor a part needs: its shape and how a random model fills it."""
     shape: tuple
-    init: str = "matrix"            # "matrix", "norm", "embedding": which sigma; "zeros"; "ones"
+    init: str = "matrix"            # "matrix", "norm", "embedding": which sigma; "gain": one plus "norm"; "zeros"; "ones"
     dtype: str = "float"            # "float": kept as stored (bf16, or fp32 if stored so); "int": int32 table
 
 
@@ -24,7 +24,7 @@ class LayerSpec:
     """One layer: the arrangement (block) and the parts it arranges."""
     block: PartRef
     mixer: PartRef
-    feed_forward: PartRef
+    feed_forward: Optional[PartRef]  # None: the layer has a mixer only
     norm: PartRef                    # built once for every norm site the block declares ...
     prefixes: Dict[str, str]         # site name of the block -> checkpoint prefix
     norms: Optional[Dict[str, PartRef]] = None    # ... unless a site is named here with a norm of its own

@@ -18,6 +18,11 @@ step (`forward`).  Interfaces:
                names the norm the block applies to the stream first (or None); the block that ran
                before may already have applied it (`normed`), fused into its last add, and this block
                may do the same for the next one (`next_norm` -> `normed_next`, else None).
+               state_specs() -> {name: StateSpec} of what the block's own operations keep per sequence between
+               steps (`ctx.cache.entry_state(ctx.entry, name)`); inner_parts() -> {site: part} of further parts
+               with tensors of their own that the block builds (a convolution in front of a sub-layer).
+  Conv         state_spec() -> StateSpec | None;  forward(ctx, stream, state) -> rows: what a sub-layer reads
+               of the fp32 stream when a short causal convolution over time stands in front of it.
   Embedding    forward(ctx, tokens) -> fp32 stream;  Head  forward(ctx, rows) -> fp32 logits.
 
 `ctx` is the step's StepContext: batch geometry on the device, the kernels
@@ -77,7 +82,21 @@ class Block(Part):
     def entry_norm(self):
         return None
 
+    def state_specs(self):
+        return {}
+
+    def inner_parts(self):
+        return {}
+
     def forward(self, ctx, stream, site, normed=None, next_norm=None):
+        raise NotImplementedError
+
+
+class Conv(Part):
+    def state_spec(self):
+        return None
+
+    def forward(self, ctx, stream, state):
         raise NotImplementedError
 
 

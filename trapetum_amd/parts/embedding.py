@@ -12,38 +12,44 @@ from .base import Embedding, Head
 
 
 class ScaledEmbedding(Embedding):
-    def __init__(self, vocab_size, hidden_size, scale):
+    def __init__(self, vocab_size, hidden_size, scale, tensor="weight"):
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.scale = float(scale)
+        self.tensor = tensor             # the table's local name ("" when the prefix is the whole name)
 
     def tensor_specs(self):
-        return {"weight": TensorSpec((self.vocab_size, self.hidden_size), init="embedding")}
+        return {self.tensor: TensorSpec((self.vocab_size, self.hidden_size), init="embedding")}
 
     def bind(self, tensors, rt):
         self.rt = rt
-        self.table = rt.matrix(tensors["weight"])
+        self.table = rt.matrix(tensors[self.tensor])
 
     def forward(self, ctx, tokens):
         return ctx.ops.embed_rows(tokens, self.table, self.scale)
 
 
 class LinearHead(Head):
-    def __init__(self, vocab_size, hidden_size, softcap=None):
+    def __init__(self, vocab_size, hidden_size, softcap=None, scale=None, tensor="weight"):
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.softcap = softcap
+        self.scale = None if scale is None or float(scale) == 1.0 else float(scale)     # logits = (rows @ table^T) * scale
+        self.tensor = tensor
 
     def tensor_specs(self):
-        return {"weight": TensorSpec((self.vocab_size, self.hidden_size), init="embedding")}
+        return {self.tensor: TensorSpec((self.vocab_size, self.hidden_size), init="embedding")}
 
     def bind(self, tensors, rt):
         self.rt = rt
-        self.weight = rt.matrix(tensors["weight"])
+        self.weight = rt.matrix(tensors[self.tensor])
 
     def forward(self, ctx, rows):
         import torch
-        return ctx.ops.linear(rows, self.weight, torch.float32, softcap=self.softcap)
+        logits = ctx.ops.linear(rows, self.weight, torch.float32, softcap=self.softcap)
+        if self.scale is not None:
+            ctx.ops.scale_rows(logits, self.scale)
+        return logits
 
 
 register_part("embedding", "scaled_embedding", ScaledEmbedding)

@@ -1,0 +1,52 @@
+"""A mixture of experts: a router picks `top` of `n_experts` small gated feed-forward layers for every token.
+
+Router: z = W_router h in fp32, s = softmax(z) over all experts; the `top` largest scores choose the experts and
+weigh their outputs as they are (renormalize=True divides them by their sum).  Expert (no biases):
+g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), y = g * sigmoid(alpha g) * (u + 1), output W_down y.
+The step's (token, expert) pairs are sorted by expert on the device, so that each expert's matrices are read by one
+run of row tiles, and the weighted sum over a token's experts is formed in fp32 in a fixed order.
+"""
+from ..models.spec import TensorSpec
+from ..registry import register_part
+from .base import FeedForward
+
+
+class RoutedExperts(FeedForward):
+    def __init__(self, hidden_size, intermediate_size, n_experts, top, limit, gate_alpha=1.702, up_shift=1.0,
+                 renormalize=False, router="router", expert="e{}.", tensors=("gate", "up", "down")):
+        if not 0 < top <= n_experts:
+            raise ValueError(f"{top} of {n_experts} experts cannot be chosen")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.n_experts, self.top = int(n_experts), int(top)
+        self.limit, self.gate_alpha, self.up_shift = float(limit), float(gate_alpha), float(up_shift)
+        self.renormalize = bool(renormalize)
+        self.router_name, self.expert_name, self.names = router, expert, tuple(tensors)
+
+    def tensor_specs(self):
+        d, i = self.hidden_size, self.intermediate_size
+        specs = {self.router_name: TensorSpec((self.n_experts, d))}
+        g, u, dn = self.names
+        for e in range(self.n_experts):
+            p = self.expert_name.format(e)
+            specs.update({p + g: TensorSpec((i, d)), p + u: TensorSpec((i, d)), p + dn: TensorSpec((d, i))})
+        return specs
+
+    def bind(self, tensors, rt):
+        import torch
+        self.rt = rt
+        g, u, dn = self.names
+        ex = [self.expert_name.format(e) for e in range(self.n_experts)]
+        self.w_router = rt.matrix(tensors[self.router_name])
+        # [experts, 2 ff, width]: an expert's gate rows, then its up rows; [experts, width, ff]
+        self.w_gate_up = rt.matrix(torch.stack([torch.cat([tensors[p + g], tensors[p + u]], dim=0) for p in ex]).contiguous())
+        self.w_down = rt.matrix(torch.stack([tensors[p + dn] for p in ex]).contiguous())
+
+    def forward(self, ctx, x):
+        import torch
+        ops = ctx.ops
+        logits = ops.linear(x, self.w_router, torch.float32)        # fp32 sums of exact products
+        chosen, weights = ops.route_top(logits, self.top, self.renormalize)
+        return ops.expert_ffn(x, chosen, weights, self.w_gate_up, self.w_down, self.limit, self.gate_alpha, self.up_shift)
+
+
+register_part("feed_forward", "routed_experts", RoutedExperts)

@@ -12,20 +12,23 @@ from .base import FeedForward
 
 
 class GatedMLP(FeedForward):
-    def __init__(self, hidden_size, intermediate_size, activation):
+    def __init__(self, hidden_size, intermediate_size, activation,
+                 tensors=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.activation = activation
+        self.names = tuple(tensors)      # local names of the gate, up and down matrices
 
     def tensor_specs(self):
         d, i = self.hidden_size, self.intermediate_size
-        return {"gate_proj.weight": TensorSpec((i, d)), "up_proj.weight": TensorSpec((i, d)),
-                "down_proj.weight": TensorSpec((d, i))}
+        g, u, dn = self.names
+        return {g: TensorSpec((i, d)), u: TensorSpec((i, d)), dn: TensorSpec((d, i))}
 
     def bind(self, tensors, rt):
         self.rt = rt
-        self.w_gate_up = rt.ops.pack_gate_up(rt.matrix(tensors["gate_proj.weight"]), rt.matrix(tensors["up_proj.weight"]))
-        self.w_down = rt.matrix(tensors["down_proj.weight"])
+        g, u, dn = self.names
+        self.w_gate_up = rt.ops.pack_gate_up(rt.matrix(tensors[g]), rt.matrix(tensors[u]))
+        self.w_down = rt.matrix(tensors[dn])
 
     def forward(self, ctx, x):
         act = ctx.ops.gated_linear(x, self.w_gate_up, self.intermediate_size, self.activation, ctx.dtype)

@@ -1,0 +1,113 @@
+"""Attention through a latent: one small vector per token is cached, and every head's keys and values are products of it.
+
+Per token the layer caches c = rmsnorm(W_dkv h)[:rank] * w_norm (the latent) and r = rope(W_dkv h)[rank:] (one rotated
+key part shared by all heads).  Head h has queries [q_n | q_r] = W_q h (q_r rotated like r), keys [W_uk,h c | r] and
+values W_uv,h c; score = (q_n . W_uk,h c + q_r . r) * scale, causal softmax in fp32, output W_o over the heads.
+
+Neither keys nor values are ever formed: q_n . (W_uk,h c) = (W_uk,h^T q_n) . c, so the query is carried into the
+latent's space (one small product per head), the attention runs over the cached rows [r | c] themselves as one kv
+head of rope_dim + rank elements that every query head shares, with the row serving as key and as value, and each
+head's weighted sum of latents goes through W_uv,h afterwards.  The attention kernels are the ones grouped-query
+attention uses (its `k` and `v` pools are one tensor here); the rotated part stands first in a row because those
+kernels rotate a head's leading elements.  A step's cost is then one read of rope_dim + rank elements per cached
+token for all heads, instead of heads * (dim + vdim).
+
+A run with `own_latent=False` has no W_dkv: it attends over what the run named by its schedule entry's `cache_of`
+cached (and, in the step that caches them, over that run's rows of this step), with its own queries, W_uk, W_uv, W_o.
+"""
+from ..cache.store import TokenSpec
+from ..models.spec import TensorSpec
+from ..registry import build_part, register_part
+from .base import Mixer
+
+
+class LatentAttention(Mixer):
+    def __init__(self, hidden_size, num_heads, nope_dim, rope_dim, value_dim, latent_rank, scale, latent_eps,
+                 position=("none", {}), own_latent=True,
+                 tensors=("q", "dkv", "dkv.norm", "uk", "uv", "o")):
+        self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
+        self.nope_dim, self.rope_dim, self.value_dim, self.rank = int(nope_dim), int(rope_dim), int(value_dim), int(latent_rank)
+        self.scale = float(scale)
+        self.latent_eps = float(latent_eps)
+        self.own_latent = bool(own_latent)
+        self.position = build_part("position", position)
+        if self.position.rotary_dim > self.rope_dim:
+            raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds the rotated part of {self.rope_dim}")
+        if self.position.rotary_dim and self.position.pairing != "halves":
+            raise ValueError("the latent's rotation pairs halves; no kernel turns neighbours here")
+        self.names = dict(zip(("q", "dkv", "dkv_norm", "uk", "uv", "o"), tensors))
+
+    @property
+    def row(self):
+        """Elements of a cached row: the rotated key part, then the latent."""
+        return self.rope_dim + self.rank
+
+    def tensor_specs(self):
+        n, d, H = self.names, self.hidden_size, self.num_heads
+        specs = {n["q"]: TensorSpec((H * (self.nope_dim + self.rope_dim), d)),
+                 n["uk"]: TensorSpec((H * self.nope_dim, self.rank)), n["uv"]: TensorSpec((H * self.value_dim, self.rank)),
+                 n["o"]: TensorSpec((d, H * self.value_dim))}
+        if self.own_latent:
+            specs[n["dkv"]] = TensorSpec((self.rank + self.rope_dim, d))
+            specs[n["dkv_norm"]] = TensorSpec((self.rank,), init="gain")
+        return specs
+
+    def cache_spec(self):
+        return TokenSpec.of(None, latent=(1, self.row))
+
+    def bind(self, tensors, rt):
+        import torch
+        self.rt = rt
+        n, H, dn, dr, dv, R = self.names, self.num_heads, self.nope_dim, self.rope_dim, self.value_dim, self.rank
+        # queries head by head as [rotated | unrotated], the down-projection as [rotated key part | latent]: the order
+        # of a cached row, and of the query that meets it
+        wq = tensors[n["q"]].reshape(H, dn + dr, -1)
+        wq = torch.cat([wq[:, dn:], wq[:, :dn]], dim=1).reshape(H * (dn + dr), -1)
+        if self.own_latent:
+            wd = tensors[n["dkv"]]
+            self.w_in = rt.matrix(torch.cat([wq, wd[R:], wd[:R]], dim=0).contiguous())
+            self.latent_gain = tensors[n["dkv_norm"]].float().contiguous()
+        else:
+            self.w_in = rt.matrix(wq.contiguous())
+            self.latent_gain = None
+        self.w_absorb = rt.matrix(tensors[n["uk"]].reshape(H, dn, R).transpose(1, 2).contiguous())     # [H, rank, dim]
+        self.w_up = rt.matrix(tensors[n["uv"]].reshape(H, dv, R).contiguous())                         # [H, vdim, rank]
+        self.w_o = rt.matrix(tensors[n["o"]])
+        self.inv_freq = self.position.inv_freq(rt.device)
+
+    def forward(self, ctx, x, site):
+        ops = ctx.ops
+        H, dn, dr, dv, R, row = self.num_heads, self.nope_dim, self.rope_dim, self.value_dim, self.rank, self.row
+        owns = ctx.cache_owner == ctx.entry
+        if owns != self.own_latent:
+            raise ValueError("a latent attention without a down-projection must read another run's cache, and one with it its own")
+        if site.spec.shape_of("latent") != (1, row):
+            raise ValueError(f"the cache read here keeps rows of {site.spec.shape_of('latent')}, this layer needs (1, {row})")
+        table = ctx.page_table(site.group_index)
+        pool = site.tensor("latent")                              # [pages, 1, page, rope_dim + rank]
+        rows_cap = site.rows_cap or 0
+        m = x.shape[0]
+        proj = ops.linear(x, self.w_in, ctx.dtype)                # [M, H (dr + dn) (+ dr + rank)]
+        # rotations, the latent's norm and the cache write in one launch: the queries' rotated parts go to their
+        # places in q, the step's rows [r | c] to `mine` and into the cache
+        q, mine = ops.latent_prepare(proj, H, dn, dr, R, self.latent_gain, self.latent_eps, self.inv_freq,
+                                     self.position.rotary_dim, ctx.row_seq, ctx.row_pos, ctx.new_len, table, pool,
+                                     rows_cap, own=owns, out_dtype=ctx.dtype)
+        ops.head_linear(proj[:, :H * (dr + dn)].view(m, H, dr + dn)[:, :, dr:], self.w_absorb, q.view(m, H, row)[:, :, dr:])
+        if ctx.mode == "decode":
+            out = ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, rows_cap, self.scale, 0.0, 0,
+                                       ctx.dtype, max_keys=ctx.max_rows_visible(site))
+        else:
+            if owns:
+                ctx.offer_step_rows(latent=mine)
+            else:
+                mine = ctx.step_rows_of(ctx.cache_owner)["latent"]
+            extend = ctx.mode == "extend"
+            out = ops.attention_prefill(q, mine, mine, H, 1, row, ctx.cu_rows, ctx.max_count, self.scale, 0.0, 0, ctx.dtype,
+                                        row_seq=ctx.row_seq, row_pos=ctx.row_pos,
+                                        cached=(ctx.new_len, table, pool, pool, rows_cap) if extend else None)
+        heads = ops.head_linear(out.view(m, H, row)[:, :, dr:], self.w_up, None)      # [M, H, vdim]
+        return ops.linear(heads.view(m, H * dv), self.w_o, ctx.dtype, defer=True)
+
+
+register_part("mixer", "latent_attention", LatentAttention)

@@ -2,7 +2,7 @@
 
 Architectures: config.json["architectures"][0] -> (configuration class, function
 from a configuration to a ModelSpec).  Parts: kind of part ("mixer",
-"feed_forward", "norm", "position", "block", "embedding", "head") and a name
+"feed_forward", "norm", "position", "block", "conv", "embedding", "head") and a name
 -> the class that implements it.  The reference dispatches by file magic to
 one loader and one binary per architecture (runtime/src/lib.rs:1060-1062,
 :4567); here a model is described as data and assembled from registered parts,
@@ -13,7 +13,7 @@ from .config.base import ConfigError, architecture_name, read_config_json
 _ARCHITECTURES = {}
 _PARTS = {}
 
-PART_KINDS = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+PART_KINDS = ("mixer", "feed_forward", "norm", "position", "block", "conv", "embedding", "head")
 
 
 class Architecture:

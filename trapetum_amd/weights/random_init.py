@@ -53,13 +53,14 @@ class RandomWeights:
             return torch.zeros(ts.shape, dtype=self.store_dtype)
         if ts.init == "ones":
             return torch.ones(ts.shape, dtype=self.store_dtype)
-        sigma = self.sigma_norm if ts.init == "norm" else self.sigma
+        sigma = self.sigma_norm if ts.init in ("norm", "gain") else self.sigma
+        shift = 1.0 if ts.init == "gain" else 0.0          # a gain that is used as stored lies around one
         if self.draw_on is not None:
             gd = torch.Generator(device=self.draw_on).manual_seed(_seed_for(self.seed, name))
             t = torch.empty(ts.shape, dtype=torch.float32, device=self.draw_on).normal_(0.0, 1.0, generator=gd)
-            return (t * sigma).to(self.store_dtype)
+            return (t * sigma + shift).to(self.store_dtype)
         t = torch.empty(ts.shape, dtype=torch.float32).normal_(0.0, 1.0, generator=g)
-        return (t * sigma).to(self.store_dtype)
+        return (t * sigma + shift).to(self.store_dtype)
 
 
 def write_model_folder(config, folder, seed, sigma=0.02, sigma_norm=0.1, store_dtype="bfloat16"):
