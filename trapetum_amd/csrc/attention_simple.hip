@@ -1,4 +1,4 @@
-// Plain attention kernel for any dtype, head size up to 256 and any grouping: one wave per (row, query head),
+// Plain attention kernel for any dtype, head size up to 1024 and any grouping: one wave per (row, query head),
 // keys visited one after the other in position order with a running softmax.
 //
 // It is the float32 path's attention for prefill and decode alike (the same instruction sequence per key in
@@ -22,7 +22,8 @@ struct AttnSimpleArgs {
     int H, KV, hd; float scale, cap; int window; int paged;
 };
 
-template <typename T>
+// NJ: elements of a head a lane holds (head sizes up to 64 NJ)
+template <typename T, int NJ>
 __global__ void __launch_bounds__(64)
 attn_simple_k(AttnSimpleArgs a) {
     const int h = blockIdx.y, r = blockIdx.x, lane = threadIdx.x;
@@ -36,9 +37,9 @@ attn_simple_k(AttnSimpleArgs a) {
     }
     const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
     const T* q = (const T*)a.q + (size_t)r * a.q_stride + (size_t)h * a.hd;
-    float qv[4], o[4];
+    float qv[NJ], o[NJ];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < NJ; j++) {
         const int d = lane + 64 * j;
         qv[j] = d < a.hd ? ld_f32(q + d) : 0.f;
         o[j] = 0.f;
@@ -46,7 +47,7 @@ attn_simple_k(AttnSimpleArgs a) {
     float m = -INFINITY, l = 0.f;
     // a key's row and value row are fetched while the two keys before it are worked on (the arithmetic per key, and
     // its order, stay as they are: the loop would otherwise pay a trip to memory, or two through the page table, per key)
-    auto fetch = [&](int t, float (&kk)[4], float (&vv)[4]) {
+    auto fetch = [&](int t, float (&kk)[NJ], float (&vv)[NJ]) {
         t = t < p ? t : p;                               // past the last key: a row that exists, never used
         const T *kp, *vp;
         if (t < start) {
@@ -61,7 +62,7 @@ attn_simple_k(AttnSimpleArgs a) {
             vp = (const T*)a.v + row * a.v_stride + (size_t)g * a.hd;
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < NJ; j++) {
             const int d = lane + 64 * j;
             const int dc = d < a.hd ? d : 0;
             const float kx = ld_f32(kp + dc), vx = ld_f32(vp + dc);
@@ -69,20 +70,20 @@ attn_simple_k(AttnSimpleArgs a) {
             vv[j] = d < a.hd ? vx : 0.f;
         }
     };
-    auto use = [&](const float (&kk)[4], const float (&vv)[4]) {
+    auto use = [&](const float (&kk)[NJ], const float (&vv)[NJ]) {
         float part = 0.f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) part = fmaf(qv[j], kk[j], part);
+        for (int j = 0; j < NJ; j++) part = fmaf(qv[j], kk[j], part);
         float s = wave_sum(part) * a.scale;
         if (a.cap > 0.f) s = softcap_f(s, a.cap);
         const float m_new = fmaxf(m, s);
         const float alpha = expf(m - m_new), pr = expf(s - m_new);
         l = l * alpha + pr;
 #pragma unroll
-        for (int j = 0; j < 4; j++) o[j] = o[j] * alpha + pr * vv[j];
+        for (int j = 0; j < NJ; j++) o[j] = o[j] * alpha + pr * vv[j];
         m = m_new;
     };
-    float k0[4], v0[4], k1[4], v1[4], k2[4], v2[4];
+    float k0[NJ], v0[NJ], k1[NJ], v1[NJ], k2[NJ], v2[NJ];
     fetch(lo, k0, v0);
     fetch(lo + 1, k1, v1);
     for (int t = lo; t <= p; t += 3) {
@@ -98,7 +99,7 @@ attn_simple_k(AttnSimpleArgs a) {
     T* out = (T*)a.out + ((size_t)r * a.H + h) * a.hd;
     const float inv = 1.f / l;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < NJ; j++) {
         const int d = lane + 64 * j;
         if (d < a.hd) st_f32(out + d, o[j] * inv);
     }
@@ -107,12 +108,15 @@ attn_simple_k(AttnSimpleArgs a) {
 static int launch(const AttnSimpleArgs& a, int dtype, int M, hipStream_t s) {
     TP_REQUIRE(M > 0 && a.H > 0 && a.KV > 0 && a.hd > 0, "attention: empty shape rows=%d heads=%d kv=%d head_dim=%d", M, a.H, a.KV, a.hd);
     TP_REQUIRE(a.H % a.KV == 0, "attention: %d query heads are no multiple of %d kv heads", a.H, a.KV);
-    TP_REQUIRE(a.hd <= 256, "attention (plain kernel): head_dim %d exceeds 256", a.hd);
+    TP_REQUIRE(a.hd <= 1024, "attention (plain kernel): head_dim %d exceeds 1024", a.hd);
     TP_REQUIRE(a.H <= 65535, "attention (plain kernel): %d heads exceed one launch (65535)", a.H);
     dim3 grid(M, a.H);
-    if (dtype == TP_BF16) attn_simple_k<bf16_t><<<grid, 64, 0, s>>>(a);
-    else if (dtype == TP_F32) attn_simple_k<float><<<grid, 64, 0, s>>>(a);
-    else return tp_fail("attention: unknown dtype %d", dtype);
+    if (dtype != TP_BF16 && dtype != TP_F32) return tp_fail("attention: unknown dtype %d", dtype);
+#define TP_ATTN_SIMPLE(NJ) do { if (dtype == TP_BF16) attn_simple_k<bf16_t, NJ><<<grid, 64, 0, s>>>(a); else attn_simple_k<float, NJ><<<grid, 64, 0, s>>>(a); } while (0)
+    if (a.hd <= 256) TP_ATTN_SIMPLE(4);
+    else if (a.hd <= 512) TP_ATTN_SIMPLE(8);
+    else TP_ATTN_SIMPLE(16);
+#undef TP_ATTN_SIMPLE
     return tp_check_launch("attention (plain kernel)");
 }
 

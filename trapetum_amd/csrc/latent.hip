@@ -46,7 +46,7 @@ latent_prepare_k(const T* __restrict__ proj, long proj_stride, int H, int dn, in
             keep = pos + rows_cap >= new_len[seq];       // else a later row of this step takes the same ring row
             at = pos % rows_cap;
         }
-        const int pg = keep ? table[(size_t)seq * table_w + at / page] : -1;
+        const int pg = keep && at / page < table_w ? table[(size_t)seq * table_w + at / page] : -1;     // a table too narrow for the position caches nothing
         if (pg >= 0) dst = pool + ((size_t)pg * page + at % page) * row;
     }
     T* mr = mine + (size_t)r * row;
