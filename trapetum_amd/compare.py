@@ -1,0 +1,263 @@
+"""Two designs side by side at equal layer sizes: Golepel next to Gemma-2, random weights, one MI355X.
+
+    python bench.py --compare golepel [--sizes 2b|9b] [--layers L] [--steps K] [--warmup W]
+
+For each design: tokens per second of a prefill of 2,048 tokens and of the generation loop's decode steps at batch 8
+and 1 (HIP graphs, greedy choice on the device), and the time of the kernels a step spends its time in, one by one at
+the same shapes, with their share of the HBM or matrix peak (`measure.time_kernels` for Gemma-2, `time_golepel_kernels`
+here).  One JSON line.  The Golepel sizes follow the Gemma-2 size of the same name: its width, vocabulary and number
+of layers; 16 heads of 128 unrotated and 64 rotated elements, values of 128, a latent of 192 (a cached row of 256
+elements, against Gemma-2's 2 x 4 x 256 at 2B); every second layer reads the cache of the layer before it; the
+feed-forward alternates in pairs between a dense layer of Gemma's width and 8 experts of half that width, 2 chosen,
+so that a token passes through as many feed-forward weights in either.
+"""
+import json
+import sys
+import time
+
+from .measure import CONTEXT, OTHER_SIZES, PEAK_FLOPS, PEAK_HBM_GBS, PREFILL_TOKENS, SIZES, time_kernels
+
+
+def golepel_config(which, layers=0):
+    from .config import GolepelConfig
+    g = dict(SIZES, **OTHER_SIZES[which])
+    n = layers or g["num_hidden_layers"]
+    D, I = g["hidden_size"], g["intermediate_size"]
+    out = []
+    for i in range(n):
+        mixer = {"heads": 16, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5,
+                 "rot": {"base": 10000.0, "dims": 64}}
+        if i % 2:
+            mixer["kv_from"] = i - 1
+        if i % 4 < 2:
+            mlp = {"kind": "dense", "ff": I}
+        else:
+            mlp = {"kind": "moe", "expert": {"ff": I // 2, "limit": 7.0}, "router": {"experts": 8, "top": 2}}
+        out.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
+    return GolepelConfig.from_dict({"architecture": "Golepel", "vocab": g["vocab_size"], "width": D, "logit_scale": 1.0,
+                                    "norm": {"eps": 1e-6, "groups": 2}, "canon": {"taps": 4}, "layers": out})
+
+
+def gemma_config(which, layers=0):
+    from .config import Gemma2Config
+    g = dict(SIZES, **OTHER_SIZES[which])
+    return Gemma2Config.from_kwargs(**dict(g, num_hidden_layers=layers or g["num_hidden_layers"]))
+
+
+class Run:
+    """One design's engine and the two things timed on it."""
+
+    def __init__(self, cfg, rows, most_tokens, name):
+        import torch
+        from .engine import Engine
+        from .sampling import Sampler, SamplingParams
+        t0 = time.time()
+        self.cfg, self.name = cfg, name
+        self.engine = Engine.from_config(cfg, seed=2, sigma=0.02, dtype="bfloat16", draw_on_device=True,
+                                         max_tokens_in_cache=most_tokens, max_context=CONTEXT, max_batch=rows)
+        self.model, self.cache = self.engine.model, self.engine.cache
+        self.sampler = Sampler(self.model.rt, SamplingParams())
+        self.gen = torch.Generator().manual_seed(2)
+        torch.cuda.synchronize()
+        self.weight_bytes = sum(t.numel() * 2 for t in self._tensors())
+        print(f"[compare] {name} ready in {time.time() - t0:.1f}s, {self.weight_bytes / 1e9:.2f} GB of weights", file=sys.stderr, flush=True)
+
+    def _tensors(self):
+        import math
+        return [type("T", (), {"numel": lambda self, s=ts.shape: math.prod(s)})() for ts in self.model.tensor_layout().values()]
+
+    def prompts(self, lengths):
+        import torch
+        return [torch.randint(0, self.cfg.vocab_size, (n,), generator=self.gen).tolist() for n in lengths]
+
+    def prefill(self, tokens=PREFILL_TOKENS):
+        import torch
+
+        def once():
+            s = self.cache.acquire()
+            toks = self.prompts([tokens])[0]
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            self.model.step(self.cache, [s], toks, counts=[tokens])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            self.cache.release(s)
+            return dt
+        once()
+        return min(once() for _ in range(3))
+
+    def decode(self, lengths, steps, warmup):
+        import torch
+        from .engine.generate import BatchRun
+        items = [(i, p, i) for i, p in enumerate(self.prompts(lengths))]
+        run = BatchRun(self.model, self.cache, items, 1 << 30, self.sampler, 0, set(), graphs=self.engine.graphed)
+        try:
+            run.prefill()
+            for _ in range(warmup):
+                run.advance()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(steps):
+                run.advance()
+            torch.cuda.synchronize()
+            return time.perf_counter() - t
+        finally:
+            run.close()
+
+    def close(self):
+        import torch
+        del self.engine, self.model, self.cache, self.sampler
+        torch.cuda.empty_cache()
+
+
+def time_golepel_kernels(engine, cfg, batch, context, prefill_tokens):
+    """Microseconds of Golepel's kernels at a decode step of `batch` sequences over `context` cached tokens and at a
+    prefill of `prefill_tokens`, each called once per layer on that layer's own weights, replayed from a HIP graph.
+    {name: {"us", "GB/s" | "TFLOP/s", "frac"}}."""
+    import torch
+    from .engine.batch import StepContext
+    model, ops, dev = engine.model, engine.model.rt.ops, engine.model.rt.device
+    bf = torch.bfloat16
+    blocks = [l.block for l in model.layers]
+    own = [b for b in blocks if b.mixer.own_latent]
+    moe = [b for b in blocks if hasattr(b.feed_forward, "w_router")]
+    dense = [b for b in blocks if hasattr(b.feed_forward, "w_gate_up") and not hasattr(b.feed_forward, "w_router")]
+    mx = own[0].mixer
+    H, dn, dr, dv, R, row, D = mx.num_heads, mx.nope_dim, mx.rope_dim, mx.value_dim, mx.rank, mx.row, cfg.hidden_size
+    out = {}
+
+    def timed(name, calls, bytes_each=None, flops_each=None):
+        calls = calls * max(1, -(-24 // len(calls)))
+        calls[0]()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for f in calls:
+                    f()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        best = float("inf")
+        for _ in range(4):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b.record()
+            b.synchronize()
+            best = min(best, a.elapsed_time(b) * 1e3 / len(calls))
+        r = {"us": round(best, 2)}
+        if bytes_each is not None:
+            r["GB/s"] = round(bytes_each / best / 1e3, 1)
+            r["frac"] = round(bytes_each / best / 1e3 / PEAK_HBM_GBS, 4)
+        elif flops_each is not None:
+            r["TFLOP/s"] = round(flops_each / best / 1e6, 1)
+            r["frac"] = round(flops_each / (best * 1e-6) / PEAK_FLOPS["bfloat16"], 4)
+        out[name] = r
+
+    cache = engine.cache
+    for rows, tag in ((batch, f"decode_b{batch}"), (prefill_tokens, f"prefill_{prefill_tokens}")):
+        decode = rows == batch
+        slots = [cache.acquire() for _ in range(batch if decode else 1)]
+        try:
+            for s in slots:
+                cache.grow(s, context if decode else rows)
+            counts = [1] * batch if decode else [rows]
+            starts = [context - 1] * batch if decode else [0]
+            ctx = StepContext(model.rt, cache, slots, counts, starts, [])
+            site = cache.site(0)
+            table, pool = ctx.page_table(site.group_index), site.tensor("latent")
+            stream = torch.randn((rows, D), device=dev)
+            x = torch.randn((rows, D), device=dev).to(bf)
+            taps = cfg.canon_taps
+            state = cache.entry_state(0, "mixer_conv") if taps > 1 else None
+            conv = blocks[0].convs["mixer_conv"]
+            one = lambda f, **kw: timed(f"{tag}.{kw.pop('name')}", f, **kw)
+            one([lambda: ops.causal_conv(stream, conv.w, state, ctx.slot_ids, ctx.cu_rows, ctx.row_seq, bf, one_row_each=decode)] * 16,
+                name="conv", bytes_each=rows * D * 6.0 + (0 if not decode else rows * (taps - 1) * D * 8.0))
+            elems = lambda w: float(w.numel())
+            prod = (lambda name, calls, w, m=rows: one(calls, name=name, bytes_each=2.0 * elems(w)) if decode
+                    else one(calls, name=name, flops_each=2.0 * m * elems(w)))
+            prod("in_proj", [(lambda b=b: ops.linear(x, b.mixer.w_in, bf)) for b in own], mx.w_in)
+            proj = ops.linear(x, mx.w_in, bf)
+            prep = lambda b: ops.latent_prepare(proj, H, dn, dr, R, b.mixer.latent_gain, 1e-6, b.mixer.inv_freq, b.mixer.position.rotary_dim,
+                                                ctx.row_seq, ctx.row_pos, ctx.new_len, table, pool, 0, own=True, out_dtype=bf)
+            one([(lambda b=b: prep(b)) for b in own], name="latent_prepare", bytes_each=rows * (proj.shape[1] + H * dr + 2 * row) * 2.0)
+            q, mine = prep(own[0])
+            xq = proj[:, :H * (dr + dn)].view(rows, H, dr + dn)[:, :, dr:]
+            qv = q.view(rows, H, row)[:, :, dr:]
+            prod("absorb", [(lambda b=b: ops.head_linear(xq, b.mixer.w_absorb, qv)) for b in blocks], mx.w_absorb)
+            if decode:
+                one([lambda: ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, 0, mx.scale, 0.0, 0, bf, max_keys=context)] * 8,
+                    name=f"attention_ctx{context}", bytes_each=2.0 * batch * context * row)
+            else:
+                pairs = rows * (rows + 1) / 2.0
+                one([lambda: ops.attention_prefill(q, mine, mine, H, 1, row, ctx.cu_rows, rows, mx.scale, 0.0, 0, bf)] * 4,
+                    name="attention", flops_each=4.0 * pairs * H * row)
+            o_lat = torch.randn((rows, H * row), device=dev).to(bf)
+            ov = o_lat.view(rows, H, row)[:, :, dr:]
+            prod("up", [(lambda b=b: ops.head_linear(ov, b.mixer.w_up, None)) for b in blocks], mx.w_up)
+            heads = torch.randn((rows, H * dv), device=dev).to(bf)
+            prod("o", [(lambda b=b: ops.linear(heads, b.mixer.w_o, bf, defer=True)) for b in blocks], mx.w_o)
+            if dense:
+                ff = dense[0].feed_forward
+                prod("gate_up", [(lambda b=b: ops.gated_linear(x, b.feed_forward.w_gate_up, ff.intermediate_size, "silu", bf)) for b in dense],
+                     ff.w_gate_up[:2 * ff.intermediate_size])
+                xi = torch.randn((rows, ff.intermediate_size), device=dev).to(bf)
+                prod("down", [(lambda b=b: ops.linear(xi, b.feed_forward.w_down, bf, defer=True)) for b in dense], ff.w_down)
+            if moe:
+                ff = moe[0].feed_forward
+                logits = torch.randn((rows, ff.n_experts), device=dev)
+                chosen, weights = ops.route_top(logits, ff.top)
+                one([lambda: ops.route_top(logits, ff.top)] * 16, name="route_top")
+                used = len(set(chosen.reshape(-1).tolist()))
+                per_expert = float(ff.w_gate_up[0].numel() + ff.w_down[0].numel())
+                calls = [(lambda b=b: ops.expert_ffn(x, chosen, weights, b.feed_forward.w_gate_up, b.feed_forward.w_down, ff.limit,
+                                                     ff.gate_alpha, ff.up_shift)) for b in moe]
+                if decode:
+                    one(calls, name=f"experts_{used}_used", bytes_each=2.0 * used * per_expert)
+                else:
+                    one(calls, name="experts", flops_each=2.0 * rows * ff.top * per_expert)
+            rows_b = torch.randn((rows, D), device=dev).to(bf)
+            g = torch.ones(D, device=dev)
+            one([lambda: ops.add_rms_norm(stream, rows_b, g, 1e-6, None, 0.0, bf, groups=cfg.norm_groups)] * 16, name="add_group_norm",
+                bytes_each=rows * D * (4 + 4 + 2) + 4.0 * D)
+        finally:
+            for s in slots:
+                cache.release(s)
+    return out
+
+
+def main(args):
+    import torch
+    which = args.sizes
+    steps, warmup = args.steps, max(2, args.warmup)
+    prompt, batch = args.prompt, args.batch
+    line = {"metric": f"Golepel next to Gemma-2 at {which} layer sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "dtype": "bf16", "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
+            "sizes": which, "designs": {}, "kernels": {}}
+    most = max(PREFILL_TOKENS, batch * (prompt + steps + warmup + 128)) + 1024
+    for name, cfg in (("golepel", golepel_config(which, args.layers)), ("gemma2", gemma_config(which, args.layers))):
+        run = Run(cfg, max(batch, 8), most, name)
+        pre = run.prefill()
+        d = {"layers": len(cfg.layers) if name == "golepel" else cfg.num_hidden_layers, "weights_GB": round(run.weight_bytes / 1e9, 2),
+             f"prefill_{PREFILL_TOKENS}_tok_s": round(PREFILL_TOKENS / pre, 1), f"prefill_{PREFILL_TOKENS}_ms": round(pre * 1e3, 2)}
+        for b in (batch, 1):
+            dt = run.decode([prompt] * b, steps, warmup)
+            d[f"decode_b{b}_tok_s"] = round(b * steps / dt, 1)
+            d[f"decode_b{b}_ms_per_step"] = round(dt / steps * 1e3, 4)
+        print(f"[compare] {name}: {d}", file=sys.stderr, flush=True)
+        if name == "golepel":
+            k = time_golepel_kernels(run.engine, cfg, batch, prompt + 40, PREFILL_TOKENS)
+        else:
+            k = time_kernels(run.engine, cfg, batch, prompt + 40, PREFILL_TOKENS)
+        for kn, row in k.items():
+            print(f"[compare] {name} kernel {kn}: {row}", file=sys.stderr, flush=True)
+        line["designs"][name] = d
+        line["kernels"][name] = k
+        run.close()
+    g, m = line["designs"]["golepel"], line["designs"]["gemma2"]
+    line["value"] = g[f"decode_b{batch}_tok_s"]
+    line["ratio_to_gemma2"] = {k: round(g[k] / m[k], 3) for k in g if k.endswith("tok_s")}
+    print(json.dumps(line), flush=True)
+    return 0

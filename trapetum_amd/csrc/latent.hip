@@ -2,6 +2,7 @@
 // per-head products that carry queries into the latent's space and weighted latents out of it.
 #include "common.h"
 #include "tile.h"
+#include "tile_mfma.h"
 
 // ---- a step's projections -> rotated query parts, and the rows [rope(key part) | rmsnorm(latent) * gain] ----------
 // proj row: H heads of [dr rotated | dn unrotated] query elements, then (own) [dr key part | R latent].
@@ -122,8 +123,35 @@ head_linear_k(const T* __restrict__ x, long x_row, long x_head, const T* __restr
         }
 }
 
+// the same on the matrix cores: bf16, K a multiple of 8, every head's rows starting on 16 bytes
+template <int TM>
+__global__ void __launch_bounds__(256)
+head_linear_mfma_k(const bf16_t* __restrict__ x, long x_row, long x_head, const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
+                   long o_row, long o_head, int M, int N, int K) {
+    using Tile = MfmaTile<TM, false>;
+    __shared__ typename Tile::Shared sh;
+    const int h = blockIdx.z, m0 = blockIdx.y * TM, n0 = blockIdx.x * 64;
+    const bf16_t* xh = x + (size_t)h * x_head;
+    const bf16_t* wh = w + (size_t)h * N * K;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    Tile t;
+    t.run(K,
+        [&](int m, int k) { return m0 + m < M ? *reinterpret_cast<const uint4*>(xh + (size_t)(m0 + m) * x_row + k) : zero; },
+        [&](int n, int k) { return n0 + n < N ? *reinterpret_cast<const uint4*>(wh + (size_t)(n0 + n) * K + k) : zero; }, sh);
+#pragma unroll
+    for (int i = 0; i < Tile::MI; i++)
+#pragma unroll
+        for (int j = 0; j < Tile::NJ; j++) {
+            const int m = m0 + Tile::m_of(i), n = n0 + Tile::n_of(j);
+            if (m >= M) continue;
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                if (n + v < N) out[(size_t)m * o_row + (size_t)h * o_head + n + v] = f32_to_bf16(t.acc[0][i][j][v]);
+        }
+}
+
 extern "C" int tp_head_linear(const void* x, long x_row, long x_head, const void* w, void* out, long o_row, long o_head,
-                              int dtype, int M, int H, int N, int K, void* stream) {
+                              int dtype, int M, int H, int N, int K, int plain, void* stream) {
     TP_REQUIRE(M > 0 && H > 0 && N > 0 && K > 0, "head_linear: empty shape M=%d H=%d N=%d K=%d", M, H, N, K);
     TP_REQUIRE(x && w && out, "head_linear: a null operand");
     TP_REQUIRE(x_head >= K && o_head >= N && x_row >= (long)(H - 1) * x_head + K && o_row >= (long)(H - 1) * o_head + N,
@@ -134,6 +162,11 @@ extern "C" int tp_head_linear(const void* x, long x_row, long x_head, const void
     const int TM = few ? 16 : 64;
     dim3 grid(tp_cdiv(N, 64), tp_cdiv(M, TM), H);
     TP_REQUIRE(grid.y <= 65535, "head_linear: %d rows exceed one launch", M);
+    if (dtype == TP_BF16 && !plain && K % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0) {
+        if (few) head_linear_mfma_k<16><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)out, o_row, o_head, M, N, K);
+        else head_linear_mfma_k<64><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)out, o_row, o_head, M, N, K);
+        return tp_check_launch("head_linear (matrix cores)");
+    }
 #define TP_HEAD_LINEAR(T, TMv) head_linear_k<T, TMv><<<grid, 256, 0, s>>>((const T*)x, x_row, x_head, (const T*)w, (T*)out, o_row, o_head, M, N, K)
     if (dtype == TP_BF16) { if (few) TP_HEAD_LINEAR(bf16_t, 16); else TP_HEAD_LINEAR(bf16_t, 64); }
     else if (dtype == TP_F32) { if (few) TP_HEAD_LINEAR(float, 16); else TP_HEAD_LINEAR(float, 64); }

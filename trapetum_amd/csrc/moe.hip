@@ -3,6 +3,7 @@
 // an expert gets lives on the device, and launches are sized for the worst case.
 #include "common.h"
 #include "tile.h"
+#include "tile_mfma.h"
 
 // ---- scores = softmax(logits) over all experts; the `top` largest (ties: the smaller index) and their scores --------
 // grid (rows), one wave a row; dynamic LDS: E floats
@@ -133,6 +134,54 @@ expert_linear_k(const T* __restrict__ a, const T* __restrict__ w, const int* __r
     }
 }
 
+// the same on the matrix cores: bf16, K a multiple of 8 (rows of A and W then start on 16 bytes)
+template <bool GATED, int TM>
+__global__ void __launch_bounds__(256)
+expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
+                     int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out) {
+    using Tile = MfmaTile<TM, GATED>;
+    __shared__ typename Tile::Shared sh;
+    __shared__ int rows[TM];                             // the tile's rows of A
+    int t = blockIdx.y, e = 0, lo = 0, hi = 0;
+    for (; e < E; e++) {
+        lo = first[e]; hi = first[e + 1];
+        const int tiles = (hi - lo + TM - 1) / TM;
+        if (t < tiles) break;
+        t -= tiles;
+    }
+    if (e == E) return;
+    const int p0 = lo + t * TM, n0 = blockIdx.x * 64;
+    if (threadIdx.x < TM) {
+        const int p = p0 + threadIdx.x;
+        rows[threadIdx.x] = p < hi ? (GATED ? order[p] / top : p) : -1;
+    }
+    __syncthreads();
+    const bf16_t* we = w + (size_t)e * (GATED ? 2 : 1) * N * K;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    Tile tile;
+    tile.run(K,
+        [&](int m, int k) { const int row = rows[m]; return row >= 0 ? *reinterpret_cast<const uint4*>(a + (size_t)row * K + k) : zero; },
+        [&](int n, int k) {
+            const int u = n0 + (n & 63);
+            return u < N ? *reinterpret_cast<const uint4*>(we + ((size_t)(GATED && n >= 64 ? N : 0) + u) * K + k) : zero;
+        }, sh);
+#pragma unroll
+    for (int i = 0; i < Tile::MI; i++)
+#pragma unroll
+        for (int j = 0; j < Tile::NJ; j++) {
+            const int p = p0 + Tile::m_of(i), n = n0 + Tile::n_of(j);
+            if (p >= hi) continue;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                if (n + v >= N) continue;
+                if constexpr (GATED) {
+                    const float g = fminf(tile.acc[0][i][j][v], limit), u = fminf(fmaxf(tile.acc[1][i][j][v], -limit), limit);
+                    ((bf16_t*)out)[(size_t)p * N + n + v] = f32_to_bf16(g / (1.f + expf(-alpha * g)) * (u + shift));
+                } else ((float*)out)[(size_t)p * N + n + v] = tile.acc[0][i][j][v];
+            }
+        }
+}
+
 // ---- out[m] = sum_k weight[m, k] * pair_out[place[m top + k]], k ascending, float32.  grid (rows, column blocks) ------
 __global__ void __launch_bounds__(256)
 expert_combine_k(const float* __restrict__ pair_out, const int* __restrict__ place, const float* __restrict__ weight, int top, int D,
@@ -154,7 +203,7 @@ extern "C" long tp_expert_ffn_workspace_bytes(int dtype, int M, int top, int E, 
 
 extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* chosen, const float* weight, int top, int E, int F,
                              const void* w_gate_up, const void* w_down, float limit, float alpha, float shift,
-                             void* workspace, long workspace_bytes, float* out, void* stream) {
+                             void* workspace, long workspace_bytes, float* out, int plain, void* stream) {
     TP_REQUIRE(M > 0 && D > 0 && top > 0 && E > 0 && F > 0, "expert_ffn: empty shape M=%d D=%d top=%d E=%d F=%d", M, D, top, E, F);
     TP_REQUIRE(x && chosen && weight && w_gate_up && w_down && workspace && out, "expert_ffn: a null operand");
     TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F32, "expert_ffn: unknown dtype %d", dtype);
@@ -176,6 +225,19 @@ extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* 
     TP_REQUIRE(row_tiles <= 65535, "expert_ffn: %d row tiles exceed one launch", row_tiles);
 #define TP_EXPERT(T, G, TMv, Nv, Kv, A, W, O) expert_linear_k<T, G, TMv><<<dim3(tp_cdiv(Nv, 64), row_tiles), 256, 0, s>>>( \
         (const T*)(A), (const T*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O)
+#define TP_EXPERT_MFMA(G, TMv, Nv, Kv, A, W, O) expert_linear_mfma_k<G, TMv><<<dim3(tp_cdiv(Nv, 64), row_tiles), 256, 0, s>>>( \
+        (const bf16_t*)(A), (const bf16_t*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O)
+    const bool cores = dtype == TP_BF16 && !plain && D % 8 == 0 && F % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w_gate_up % 16 == 0 &&
+                       (uintptr_t)w_down % 16 == 0;
+    if (cores) {
+        if (few) TP_EXPERT_MFMA(true, 16, F, D, x, w_gate_up, y); else TP_EXPERT_MFMA(true, 64, F, D, x, w_gate_up, y);
+        if (int rc = tp_check_launch("expert_ffn (gate, up; matrix cores)")) return rc;
+        if (few) TP_EXPERT_MFMA(false, 16, D, F, y, w_down, pair_out); else TP_EXPERT_MFMA(false, 64, D, F, y, w_down, pair_out);
+        if (int rc = tp_check_launch("expert_ffn (down; matrix cores)")) return rc;
+        expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, place, weight, top, D, out);
+        return tp_check_launch("expert_ffn (combine)");
+    }
+#undef TP_EXPERT_MFMA
     if (dtype == TP_BF16) { if (few) TP_EXPERT(bf16_t, true, 16, F, D, x, w_gate_up, y); else TP_EXPERT(bf16_t, true, 64, F, D, x, w_gate_up, y); }
     else { if (few) TP_EXPERT(float, true, 16, F, D, x, w_gate_up, y); else TP_EXPERT(float, true, 64, F, D, x, w_gate_up, y); }
     if (int rc = tp_check_launch("expert_ffn (gate, up)")) return rc;

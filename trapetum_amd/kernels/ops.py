@@ -20,10 +20,10 @@ _CORE_SIGS = {
     "tp_scale_rows": [_P, _L, _F, _P],
     "tp_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "tp_latent_prepare": [_P, _L, _I, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _P],
-    "tp_head_linear": [_P, _L, _L, _P, _P, _L, _L, _I, _I, _I, _I, _I, _P],
+    "tp_head_linear": [_P, _L, _L, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P],
     "tp_route_top": [_P, _I, _I, _I, _I, _P, _P, _P],
     "tp_expert_ffn_workspace_bytes": [_I, _I, _I, _I, _I, _I],
-    "tp_expert_ffn": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _P, _F, _F, _F, _P, _L, _P, _P],
+    "tp_expert_ffn": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _P, _F, _F, _F, _P, _L, _P, _I, _P],
     "tp_gather_rows": [_P, _P, _P, _I, _I, _I, _P],
     "tp_sum_slices": [_P, _I, _L, _P, _I, _L, _P],
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
@@ -322,7 +322,7 @@ class HipOps:
             if t.shape[2] > 1 and t.stride(2) != 1:
                 raise KernelError(f"head_linear: a head's elements must be contiguous in the {what}")
         self._call(self.lib, "tp_head_linear", x.data_ptr(), x.stride(0), x.stride(1), w.data_ptr(), out.data_ptr(),
-                   out.stride(0), out.stride(1), _code(x.dtype), m, H, N, K, self._stream())
+                   out.stride(0), out.stride(1), _code(x.dtype), m, H, N, K, 1 if self.force_linear == 1 else 0, self._stream())
         return out
 
     # ---- mixture of experts ------------------------------------------------------------------------------------
@@ -363,7 +363,7 @@ class HipOps:
         out = torch.empty((m, d), dtype=torch.float32, device=self.device)
         self._call(self.lib, "tp_expert_ffn", x.data_ptr(), _code(x.dtype), m, d, chosen.data_ptr(), weights.data_ptr(), top, e, f,
                    w_gate_up.data_ptr(), w_down.data_ptr(), float(limit), float(alpha), float(shift), ws.data_ptr(), nbytes,
-                   out.data_ptr(), self._stream())
+                   out.data_ptr(), 1 if self.force_linear == 1 else 0, self._stream())
         return out
 
     MAX_SLICED_WIDTH = 8192        # widest row `add_rms_norm` takes in K slices
