@@ -48,7 +48,7 @@ def scale_rows(x, scale):
     x *= scale
 
 
-def causal_conv(stream, w, state, slot_ids, cu_rows, row_seq, out_dtype, residual=True, one_row_each=False):
+def causal_conv(stream, w, state, slot_ids, cu_rows, row_seq, out_dtype, residual=True, one_row_each=False, w_t=None):
     """out_t = (x_t) + sum_j w[:, j] x_(t - taps + 1 + j); rows before the step come from state[slot] ([taps - 1, D],
     oldest first), which then takes the last taps - 1 rows of (state, step)."""
     taps = w.shape[1]

@@ -140,6 +140,21 @@ def test_latent_attention_part(rt, H, dn, dr, dv, R, rot):
     assert rel_l2(torch.cat(got2), want2) < tol
 
 
+@pytest.mark.parametrize("m,h,n,k,lead", [(5, 3, 32, 16, 16), (100, 4, 24, 40, 8), (700, 2, 200, 72, 0), (9, 5, 7, 12, 6), (600, 3, 50, 24, 16)])
+def test_head_linear(rt, m, h, n, k, lead):
+    """Per-head products on views of wider rows: each head's `k` elements follow `lead` others, and the output lands
+    behind `lead` elements of each head of a wider row as well."""
+    x = rnd(m, h, lead + k, seed=70).to(rt.dtype).to(DEV)
+    w = rnd(h, n, k, seed=71, scale=0.3).to(rt.dtype).to(DEV)
+    want = torch.einsum("mhk,hnk->mhn", x[:, :, lead:].double().cpu(), w.double().cpu())
+    got = rt.ops.head_linear(x[:, :, lead:], w)
+    assert got.is_contiguous() and rel_l2(got, want) < PART_TOL[rt.dtype]
+    wide = torch.full((m, h, lead + n), 7.0, dtype=rt.dtype, device=DEV)
+    rt.ops.head_linear(x[:, :, lead:], w, wide[:, :, lead:])
+    assert rel_l2(wide[:, :, lead:], want) < PART_TOL[rt.dtype]
+    assert bool((wide[:, :, :lead] == 7.0).all())
+
+
 @pytest.mark.parametrize("page,counts", [(16, (15, 1, 1, 1, 31, 2, 1, 40, 1, 1, 1, 1, 1, 2)), (64, (64, 1, 30, 1, 1, 1, 1, 1))])
 def test_latent_attention_sharp_scores(rt, page, counts):
     """Scores scaled until a softmax picks single keys, wherever they lie: a key lost or read one row off, at a page's
@@ -169,7 +184,7 @@ def test_latent_attention_sharp_scores(rt, page, counts):
 
 
 @pytest.mark.parametrize("m,d,f,e,top,limit", [(1, 64, 40, 5, 3, 0.8), (9, 50, 18, 2, 2, 0.5), (150, 96, 70, 16, 2, 1.5),
-                                               (70, 128, 33, 9, 1, 2.0), (300, 72, 24, 130, 4, 1.0)])
+                                               (70, 128, 33, 9, 1, 2.0), (300, 72, 24, 130, 4, 1.0), (650, 136, 200, 3, 2, 1.2), (5, 64, 1024, 3, 2, 1.0)])
 def test_routed_experts(rt, m, d, f, e, top, limit):
     part = build_part("feed_forward", ("routed_experts", dict(hidden_size=d, intermediate_size=f, n_experts=e, top=top, limit=limit)))
     dev, W = {}, {}

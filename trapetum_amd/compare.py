@@ -173,7 +173,7 @@ def time_golepel_kernels(engine, cfg, batch, context, prefill_tokens):
             state = cache.entry_state(0, "mixer_conv") if taps > 1 else None
             conv = blocks[0].convs["mixer_conv"]
             one = lambda f, **kw: timed(f"{tag}.{kw.pop('name')}", f, **kw)
-            one([lambda: ops.causal_conv(stream, conv.w, state, ctx.slot_ids, ctx.cu_rows, ctx.row_seq, bf, one_row_each=decode)] * 16,
+            one([lambda: ops.causal_conv(stream, conv.w, state, ctx.slot_ids, ctx.cu_rows, ctx.row_seq, bf, one_row_each=decode, w_t=conv.w_t)] * 16,
                 name="conv", bytes_each=rows * D * 6.0 + (0 if not decode else rows * (taps - 1) * D * 8.0))
             elems = lambda w: float(w.numel())
             prod = (lambda name, calls, w, m=rows: one(calls, name=name, bytes_each=2.0 * elems(w)) if decode
@@ -186,7 +186,9 @@ def time_golepel_kernels(engine, cfg, batch, context, prefill_tokens):
             q, mine = prep(own[0])
             xq = proj[:, :H * (dr + dn)].view(rows, H, dr + dn)[:, :, dr:]
             qv = q.view(rows, H, row)[:, :, dr:]
-            prod("absorb", [(lambda b=b: ops.head_linear(xq, b.mixer.w_absorb, qv)) for b in blocks], mx.w_absorb)
+            # the per-head products move rows in and out for some 70 flop a byte, far below the ridge: priced by bytes
+            one([(lambda b=b: ops.head_linear(xq, b.mixer.w_absorb, qv)) for b in blocks], name="absorb",
+                bytes_each=2.0 * (elems(mx.w_absorb) + rows * H * (dn + R)))
             if decode:
                 one([lambda: ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, 0, mx.scale, 0.0, 0, bf, max_keys=context)] * 8,
                     name=f"attention_ctx{context}", bytes_each=2.0 * batch * context * row)
@@ -196,7 +198,8 @@ def time_golepel_kernels(engine, cfg, batch, context, prefill_tokens):
                     name="attention", flops_each=4.0 * pairs * H * row)
             o_lat = torch.randn((rows, H * row), device=dev).to(bf)
             ov = o_lat.view(rows, H, row)[:, :, dr:]
-            prod("up", [(lambda b=b: ops.head_linear(ov, b.mixer.w_up, None)) for b in blocks], mx.w_up)
+            one([(lambda b=b: ops.head_linear(ov, b.mixer.w_up, None)) for b in blocks], name="up",
+                bytes_each=2.0 * (elems(mx.w_up) + rows * H * (R + dv)))
             heads = torch.randn((rows, H * dv), device=dev).to(bf)
             prod("o", [(lambda b=b: ops.linear(heads, b.mixer.w_o, bf, defer=True)) for b in blocks], mx.w_o)
             if dense:

@@ -134,6 +134,7 @@ head_linear_mfma_k(const bf16_t* __restrict__ x, long x_row, long x_head, const 
     const bf16_t* xh = x + (size_t)h * x_head;
     const bf16_t* wh = w + (size_t)h * N * K;
     const uint4 zero = make_uint4(0, 0, 0, 0);
+    const bool wide = o_row % 4 == 0 && o_head % 4 == 0 && (uintptr_t)out % 8 == 0;
     Tile t;
     t.run(K,
         [&](int m, int k) { return m0 + m < M ? *reinterpret_cast<const uint4*>(xh + (size_t)(m0 + m) * x_row + k) : zero; },
@@ -144,9 +145,17 @@ head_linear_mfma_k(const bf16_t* __restrict__ x, long x_row, long x_head, const 
         for (int j = 0; j < Tile::NJ; j++) {
             const int m = m0 + Tile::m_of(i), n = n0 + Tile::n_of(j);
             if (m >= M) continue;
+            bf16_t* dst = out + (size_t)m * o_row + (size_t)h * o_head + n;
+            if (wide && n + 3 < N) {                      // the lane's four neighbours in one store
+                uint2 o;
+                o.x = (uint32_t)f32_to_bf16(t.acc[0][i][j][0]) | ((uint32_t)f32_to_bf16(t.acc[0][i][j][1]) << 16);
+                o.y = (uint32_t)f32_to_bf16(t.acc[0][i][j][2]) | ((uint32_t)f32_to_bf16(t.acc[0][i][j][3]) << 16);
+                *reinterpret_cast<uint2*>(dst) = o;
+                continue;
+            }
 #pragma unroll
             for (int v = 0; v < 4; v++)
-                if (n + v < N) out[(size_t)m * o_row + (size_t)h * o_head + n + v] = f32_to_bf16(t.acc[0][i][j][v]);
+                if (n + v < N) dst[v] = f32_to_bf16(t.acc[0][i][j][v]);
         }
 }
 
@@ -162,6 +171,11 @@ extern "C" int tp_head_linear(const void* x, long x_row, long x_head, const void
     const int TM = few ? 16 : 64;
     dim3 grid(tp_cdiv(N, 64), tp_cdiv(M, TM), H);
     TP_REQUIRE(grid.y <= 65535, "head_linear: %d rows exceed one launch", M);
+    if (dtype == TP_BF16 && !plain && M >= 512 && K % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0) {
+        grid.y = tp_cdiv(M, 128);
+        head_linear_mfma_k<128><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)out, o_row, o_head, M, N, K);
+        return tp_check_launch("head_linear (matrix cores)");
+    }
     if (dtype == TP_BF16 && !plain && K % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0) {
         if (few) head_linear_mfma_k<16><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)out, o_row, o_head, M, N, K);
         else head_linear_mfma_k<64><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)out, o_row, o_head, M, N, K);

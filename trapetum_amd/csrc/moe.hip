@@ -134,12 +134,15 @@ expert_linear_k(const T* __restrict__ a, const T* __restrict__ w, const int* __r
     }
 }
 
-// the same on the matrix cores: bf16, K a multiple of 8 (rows of A and W then start on 16 bytes)
-template <bool GATED, int TM>
+// the same on the matrix cores: bf16, K a multiple of 8 (rows of A and W then start on 16 bytes).
+// MODE 0: 64 columns a block; 1: gated, 64 units (their gate and up rows); 2: 128 columns a block (two sets of 64).
+template <int MODE, int TM>
 __global__ void __launch_bounds__(256)
 expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
-                     int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out) {
-    using Tile = MfmaTile<TM, GATED>;
+                     int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out, int k_slice, long out_slice) {
+    constexpr bool GATED = MODE == 1;
+    constexpr int COLS = MODE == 2 ? 128 : 64;
+    using Tile = MfmaTile<TM, MODE != 0>;
     __shared__ typename Tile::Shared sh;
     __shared__ int rows[TM];                             // the tile's rows of A
     int t = blockIdx.y, e = 0, lo = 0, hi = 0;
@@ -150,7 +153,7 @@ expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
         t -= tiles;
     }
     if (e == E) return;
-    const int p0 = lo + t * TM, n0 = blockIdx.x * 64;
+    const int p0 = lo + t * TM, n0 = blockIdx.x * COLS;
     if (threadIdx.x < TM) {
         const int p = p0 + threadIdx.x;
         rows[threadIdx.x] = p < hi ? (GATED ? order[p] / top : p) : -1;
@@ -158,39 +161,72 @@ expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
     __syncthreads();
     const bf16_t* we = w + (size_t)e * (GATED ? 2 : 1) * N * K;
     const uint4 zero = make_uint4(0, 0, 0, 0);
+    // a plain product of few rows may come in K slices (grid z): slice z sums k in [z k_slice, (z + 1) k_slice) into its
+    // own copy of the output, and the consumer adds the copies in slice order
+    const int kz = blockIdx.z * k_slice, klen = min(K - kz, k_slice);
+    if (!GATED) out = (float*)out + (size_t)blockIdx.z * out_slice;
     Tile tile;
-    tile.run(K,
-        [&](int m, int k) { const int row = rows[m]; return row >= 0 ? *reinterpret_cast<const uint4*>(a + (size_t)row * K + k) : zero; },
+    tile.run(klen,
+        [&](int m, int k) { const int row = rows[m]; return row >= 0 ? *reinterpret_cast<const uint4*>(a + (size_t)row * K + kz + k) : zero; },
         [&](int n, int k) {
-            const int u = n0 + (n & 63);
-            return u < N ? *reinterpret_cast<const uint4*>(we + ((size_t)(GATED && n >= 64 ? N : 0) + u) * K + k) : zero;
+            const int u = GATED ? n0 + (n & 63) : n0 + n;          // gated: the staged rows 64 .. 127 are the units' up rows
+            return u < N ? *reinterpret_cast<const uint4*>(we + ((size_t)(GATED && n >= 64 ? N : 0) + u) * K + kz + k) : zero;
         }, sh);
 #pragma unroll
     for (int i = 0; i < Tile::MI; i++)
 #pragma unroll
         for (int j = 0; j < Tile::NJ; j++) {
-            const int p = p0 + Tile::m_of(i), n = n0 + Tile::n_of(j);
+            const int p = p0 + Tile::m_of(i);
             if (p >= hi) continue;
+            if constexpr (GATED) {
+                const int n = n0 + Tile::n_of(j);
+                bf16_t o[4];
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                if (n + v >= N) continue;
-                if constexpr (GATED) {
+                for (int v = 0; v < 4; v++) {
                     const float g = fminf(tile.acc[0][i][j][v], limit), u = fminf(fmaxf(tile.acc[1][i][j][v], -limit), limit);
-                    ((bf16_t*)out)[(size_t)p * N + n + v] = f32_to_bf16(g / (1.f + expf(-alpha * g)) * (u + shift));
-                } else ((float*)out)[(size_t)p * N + n + v] = tile.acc[0][i][j][v];
+                    o[v] = f32_to_bf16(g / (1.f + expf(-alpha * g)) * (u + shift));
+                }
+                bf16_t* dst = (bf16_t*)out + (size_t)p * N + n;
+                if ((N & 3) == 0 && n + 3 < N) {         // the lane's four neighbours in one store
+                    uint2 pk;
+                    pk.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+                    pk.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+                    *reinterpret_cast<uint2*>(dst) = pk;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) if (n + v < N) dst[v] = o[v];
+                }
+            } else {
+#pragma unroll
+                for (int set = 0; set < Tile::SETS; set++) {
+                    const int n = n0 + 64 * set + Tile::n_of(j);
+                    float* dst = (float*)out + (size_t)p * N + n;
+                    if ((N & 3) == 0 && n + 3 < N)
+                        *reinterpret_cast<float4*>(dst) = make_float4(tile.acc[set][i][j][0], tile.acc[set][i][j][1], tile.acc[set][i][j][2], tile.acc[set][i][j][3]);
+                    else {
+#pragma unroll
+                        for (int v = 0; v < 4; v++) if (n + v < N) dst[v] = tile.acc[set][i][j][v];
+                    }
+                }
             }
         }
 }
 
 // ---- out[m] = sum_k weight[m, k] * pair_out[place[m top + k]], k ascending, float32.  grid (rows, column blocks) ------
+// K slices the down product of a decode step is cut in (when the experts' width allows slices of whole steps)
+static int down_slices(int P, int F) { return (P <= 64 && F >= 1024 && F % 256 == 0) ? 4 : 1; }
 __global__ void __launch_bounds__(256)
-expert_combine_k(const float* __restrict__ pair_out, const int* __restrict__ place, const float* __restrict__ weight, int top, int D,
-                 float* __restrict__ out) {
+expert_combine_k(const float* __restrict__ pair_out, int n_slices, long slice_stride, const int* __restrict__ place,
+                 const float* __restrict__ weight, int top, int D, float* __restrict__ out) {
     const int m = blockIdx.x, d = blockIdx.y * 256 + threadIdx.x;
     if (d >= D) return;
     float acc = 0.f;
-    for (int k = 0; k < top; k++)
-        acc = __builtin_fmaf(weight[(size_t)m * top + k], pair_out[(size_t)place[(size_t)m * top + k] * D + d], acc);
+    for (int k = 0; k < top; k++) {
+        const float* src = pair_out + (size_t)place[(size_t)m * top + k] * D + d;
+        float v = src[0];
+        for (int z = 1; z < n_slices; z++) v += src[(size_t)z * slice_stride];       // the K slices of a pair's output, in slice order
+        acc = __builtin_fmaf(weight[(size_t)m * top + k], v, acc);
+    }
     out[(size_t)m * D + d] = acc;
 }
 
@@ -198,7 +234,7 @@ expert_combine_k(const float* __restrict__ pair_out, const int* __restrict__ pla
 static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 extern "C" long tp_expert_ffn_workspace_bytes(int dtype, int M, int top, int E, int F, int D) {
     const size_t P = (size_t)M * top, el = dtype == TP_BF16 ? 2 : 4;
-    return (long)(align256((2 * P + E + 1) * sizeof(int)) + align256(P * F * el) + align256(P * D * sizeof(float)));
+    return (long)(align256((2 * P + E + 1) * sizeof(int)) + align256(P * F * el) + align256(P * D * sizeof(float) * down_slices((int)P, F)));
 }
 
 extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* chosen, const float* weight, int top, int E, int F,
@@ -220,21 +256,23 @@ extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* 
     expert_sort_k<<<E, 256, 0, s>>>(chosen, P, E, order, place, first);
     if (int rc = tp_check_launch("expert_ffn (sort)")) return rc;
     const bool few = P <= 64;                            // a decode step: most runs hold a pair or two
-    const int TM = few ? 16 : 64;
+    const bool cores = dtype == TP_BF16 && !plain && D % 8 == 0 && F % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w_gate_up % 16 == 0 &&
+                       (uintptr_t)w_down % 16 == 0;
+    const bool many = cores && P >= 128 * E;             // runs of a hundred pairs and more: tiles of 128 rows
+    const int TM = few ? 16 : (many ? 128 : 64);
     const int row_tiles = tp_cdiv(P, TM) + (E < P ? E : P);
     TP_REQUIRE(row_tiles <= 65535, "expert_ffn: %d row tiles exceed one launch", row_tiles);
 #define TP_EXPERT(T, G, TMv, Nv, Kv, A, W, O) expert_linear_k<T, G, TMv><<<dim3(tp_cdiv(Nv, 64), row_tiles), 256, 0, s>>>( \
         (const T*)(A), (const T*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O)
-#define TP_EXPERT_MFMA(G, TMv, Nv, Kv, A, W, O) expert_linear_mfma_k<G, TMv><<<dim3(tp_cdiv(Nv, 64), row_tiles), 256, 0, s>>>( \
-        (const bf16_t*)(A), (const bf16_t*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O)
-    const bool cores = dtype == TP_BF16 && !plain && D % 8 == 0 && F % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w_gate_up % 16 == 0 &&
-                       (uintptr_t)w_down % 16 == 0;
+#define TP_EXPERT_MFMA(G, TMv, Nv, Kv, A, W, O, Z) expert_linear_mfma_k<G, TMv><<<dim3(tp_cdiv(Nv, (G) == 2 ? 128 : 64), row_tiles, Z), 256, 0, s>>>( \
+        (const bf16_t*)(A), (const bf16_t*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O, (Kv) / (Z), (long)P * (Nv))
     if (cores) {
-        if (few) TP_EXPERT_MFMA(true, 16, F, D, x, w_gate_up, y); else TP_EXPERT_MFMA(true, 64, F, D, x, w_gate_up, y);
+        if (few) TP_EXPERT_MFMA(1, 16, F, D, x, w_gate_up, y, 1); else if (many) TP_EXPERT_MFMA(1, 128, F, D, x, w_gate_up, y, 1); else TP_EXPERT_MFMA(1, 64, F, D, x, w_gate_up, y, 1);
         if (int rc = tp_check_launch("expert_ffn (gate, up; matrix cores)")) return rc;
-        if (few) TP_EXPERT_MFMA(false, 16, D, F, y, w_down, pair_out); else TP_EXPERT_MFMA(false, 64, D, F, y, w_down, pair_out);
+        const int zs = down_slices(P, F);
+        if (few) TP_EXPERT_MFMA(0, 16, D, F, y, w_down, pair_out, zs); else if (many) TP_EXPERT_MFMA(2, 128, D, F, y, w_down, pair_out, 1); else TP_EXPERT_MFMA(0, 64, D, F, y, w_down, pair_out, 1);
         if (int rc = tp_check_launch("expert_ffn (down; matrix cores)")) return rc;
-        expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, place, weight, top, D, out);
+        expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, zs, (long)P * D, place, weight, top, D, out);
         return tp_check_launch("expert_ffn (combine)");
     }
 #undef TP_EXPERT_MFMA
@@ -245,6 +283,6 @@ extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* 
     else { if (few) TP_EXPERT(float, false, 16, D, F, y, w_down, pair_out); else TP_EXPERT(float, false, 64, D, F, y, w_down, pair_out); }
 #undef TP_EXPERT
     if (int rc = tp_check_launch("expert_ffn (down)")) return rc;
-    expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, place, weight, top, D, out);
+    expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, 1, 0, place, weight, top, D, out);
     return tp_check_launch("expert_ffn (combine)");
 }

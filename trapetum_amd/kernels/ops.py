@@ -18,7 +18,7 @@ _CORE_SIGS = {
     "tp_rms_norm": [_P, _I, _P, _F, _P, _I, _I, _I, _I, _P],
     "tp_add_rms_norm": [_P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _I, _I, _I, _I, _P],
     "tp_scale_rows": [_P, _L, _F, _P],
-    "tp_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "tp_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "tp_latent_prepare": [_P, _L, _I, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _P],
     "tp_head_linear": [_P, _L, _L, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P],
     "tp_route_top": [_P, _I, _I, _I, _I, _P, _P, _P],
@@ -249,10 +249,11 @@ class HipOps:
             raise KernelError("scale_rows: expected a contiguous float32 tensor")
         self._call(self.lib, "tp_scale_rows", x.data_ptr(), x.numel(), float(scale), self._stream())
 
-    def causal_conv(self, stream, w, state, slot_ids, cu_rows, row_seq, out_dtype, residual=True, one_row_each=False):
+    def causal_conv(self, stream, w, state, slot_ids, cu_rows, row_seq, out_dtype, residual=True, one_row_each=False, w_t=None):
         """out[r] = (stream[r]) + sum_j w[:, j] * stream[r - (taps - 1) + j] within each sequence; the rows before the
         step are read from state[slot] (float32 [slots, taps - 1, D], oldest first), which then takes the last
-        taps - 1 rows of (state, step).  one_row_each: every sequence brings one row (one launch does both)."""
+        taps - 1 rows of (state, step).  one_row_each: every sequence brings one row (one launch does both).
+        w_t: the taps transposed, contiguous float32 [taps, D], for the kernel that takes four channels a thread."""
         self._dev(stream, w, state, slot_ids, cu_rows, row_seq)
         if stream.dtype != torch.float32 or stream.dim() != 2 or not stream.is_contiguous():
             raise KernelError("causal_conv: the stream must be contiguous float32 [rows, channels]")
@@ -266,8 +267,12 @@ class HipOps:
         if taps > 1 and (state is None or state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (taps - 1, d)
                          or not state.is_contiguous()):
             raise KernelError(f"causal_conv: the state must be contiguous float32 [slots, {taps - 1}, {d}]")
+        if w_t is not None and (w_t.dtype != torch.float32 or tuple(w_t.shape) != (taps, d) or not w_t.is_contiguous()):
+            raise KernelError(f"causal_conv: the transposed taps must be contiguous float32 [{taps}, {d}]")
+        self._dev(w_t)
         out = torch.empty((m, d), dtype=out_dtype, device=self.device)
-        self._call(self.lib, "tp_causal_conv", stream.data_ptr(), w.data_ptr(), state.data_ptr() if taps > 1 else None,
+        self._call(self.lib, "tp_causal_conv", stream.data_ptr(), w.data_ptr(), w_t.data_ptr() if w_t is not None else None,
+                   state.data_ptr() if taps > 1 else None,
                    slot_ids.data_ptr(), cu_rows.data_ptr(), row_seq.data_ptr(), out.data_ptr(), _code(out_dtype), m, n_seq, d, taps,
                    1 if residual else 0, 1 if one_row_each else 0, self._stream())
         return out

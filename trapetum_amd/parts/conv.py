@@ -26,10 +26,11 @@ class CausalConv(Conv):
     def bind(self, tensors, rt):
         self.rt = rt
         self.w = tensors[self.tensor].float().contiguous()
+        self.w_t = self.w.t().contiguous()               # [taps, channels]: neighbouring channels' taps side by side
 
     def forward(self, ctx, stream, state):
         return ctx.ops.causal_conv(stream, self.w, state, ctx.slot_ids, ctx.cu_rows, ctx.row_seq, ctx.dtype,
-                                   residual=self.residual, one_row_each=ctx.mode == "decode")
+                                   residual=self.residual, one_row_each=ctx.mode == "decode", w_t=self.w_t)
 
 
 register_part("conv", "causal_conv", CausalConv)
