@@ -293,3 +293,54 @@ def test_greedy_generation_through_the_entry_point(which, dtype, tmp_path):
     again = engine.generate(prompts[::-1], max_tokens=12, stop_ids=())       # replayed graphs, other slots
     assert again == got[::-1]
     assert engine.cache.live_slots() == []
+
+
+# ---- the programs a user runs ------------------------------------------------------------------------------------------------
+def test_command_line_and_trace_runner(tmp_path):
+    """`python -m trapetum_amd random | run | generate` and bin/trace_run on a Golepel folder: the model class comes from
+    config.json, the ids and logits are the plain implementation's."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    from . import trace_schedules as ts
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+    def run(cmd, **kw):
+        p = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=300, **kw)
+        assert p.returncode == 0, p.stderr[-2000:]
+        return p.stdout
+    cfg, init = gt.CONFIGS["P"]
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(cfg))
+    folder = tmp_path / "model"
+    module = [sys.executable, "-m", "trapetum_amd"]
+    assert "wrote" in run(module + ["random", "--config", str(config), "--out", str(folder), "--seed", str(init["seed"]),
+                                    "--sigma", str(init["sigma"]), "--sigma-norm", str(init["sigma_norm"])])
+    pcfg, pw = plain.read_folder(str(folder))
+    prompts = [random_tokens(n, pcfg["vocab"], 95 + n) for n in (6, 13)]
+    want = [plain.greedy_generate(pcfg, pw, p, 7) for p in prompts]
+    out = run(module + ["run", str(folder), "--prompt-ids", ",".join(map(str, prompts[0])), "--max-tokens", "7", "--dtype", "float32"])
+    assert out.strip() == f"continuation ids: {want[0]}"
+    ids = tmp_path / "ids.txt"
+    ids.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    out = run(module + ["generate", str(folder), "--prompts-file", str(ids), "--max-tokens", "7", "--dtype", "float32"])
+    assert [[int(t) for t in line.split()] for line in out.strip().splitlines()] == want
+    sampled = run(module + ["generate", str(folder), "--prompts-file", str(ids), "--max-tokens", "7", "--temperature", "0.8", "--seed", "5"])
+    assert sampled == run(module + ["generate", str(folder), "--prompts-file", str(ids), "--max-tokens", "7", "--temperature", "0.8", "--seed", "5"])
+    assert all(len(line.split()) == 7 for line in sampled.strip().splitlines())
+    # the trace runner: requests whole, in unequal batches, and with their last tokens one by one
+    requests = {f"r{i}": random_tokens(n, pcfg["vocab"], 20 + i) for i, n in enumerate([40, 3, 21])}
+    ref = {rid: plain.forward(pcfg, pw, t) for rid, t in requests.items()}
+    for name, steps in (("whole", ts.whole(requests)), ("tail", ts.last_one_by_one(requests, 12)), ("batches", ts.batches(requests, 3))):
+        out_dir = tmp_path / name
+        stdout = run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(folder), "--dtype", "float32", "--out", str(out_dir),
+                      "--max-tokens", str(ts.held_tokens(steps))], input="".join(json.dumps(s) + "\n" for s in steps))
+        assert [l for l in stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+        outputs = {s["step"]: np.fromfile(out_dir / f"{s['step']}.f32", dtype="<f4") for s in steps if any(e["want"] for e in s["entries"])}
+        got = ts.collect(steps, outputs, pcfg["vocab"])
+        for rid in requests:
+            assert rel_l2(torch.from_numpy(got[rid]), ref[rid]) < 2e-5, (name, rid)
