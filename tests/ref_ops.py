@@ -225,7 +225,11 @@ def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, wi
     return out.to(out_dtype)
 
 
-def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype, max_keys=None):
+def decode_splits(n, KV, hd, keys):
+    return 1
+
+
+def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype, max_keys=None, splits=None):
     n = q.shape[0]
     page = k_pool.shape[2]
     out = torch.zeros((n, H * hd), dtype=torch.float32, device=q.device)

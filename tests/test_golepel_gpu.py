@@ -109,7 +109,12 @@ def latent_part(rt, H, dn, dr, dv, R, rot, own=True, seed=0, scale=0.3):
 
 
 @pytest.mark.parametrize("H,dn,dr,dv,R,rot", [(3, 16, 16, 24, 32, 8), (1, 12, 6, 10, 20, 0), (20, 8, 8, 16, 24, 8),
-                                              (4, 32, 32, 32, 96, 32), (2, 24, 16, 8, 280, 16)])
+                                              (4, 32, 32, 32, 96, 32), (2, 24, 16, 8, 280, 16),
+                                              # cached rows of every multiple of 16 elements the matrix-core attention takes
+                                              (4, 16, 16, 16, 80, 16), (2, 16, 32, 16, 80, 32), (3, 8, 16, 8, 128, 16),
+                                              (5, 8, 16, 8, 144, 8), (2, 8, 16, 8, 160, 16), (16, 8, 32, 8, 160, 32),
+                                              (2, 8, 16, 8, 192, 16), (7, 8, 16, 8, 208, 16), (1, 8, 16, 8, 224, 16),
+                                              (16, 8, 64, 8, 192, 64), (17, 8, 16, 8, 48, 16)])
 def test_latent_attention_part(rt, H, dn, dr, dv, R, rot):
     """The mixer alone: a prompt, single tokens, a portion; then a second part without a down-projection on the same cache."""
     tol = PART_TOL[rt.dtype] * (3 if rt.dtype == torch.float32 else 1.5)

@@ -95,8 +95,12 @@ class LatentAttention(Mixer):
                                      rows_cap, own=owns, out_dtype=ctx.dtype)
         ops.head_linear(proj[:, :H * (dr + dn)].view(m, H, dr + dn)[:, :, dr:], self.w_absorb, q.view(m, H, row)[:, :, dr:])
         if ctx.mode == "decode":
+            # every slice of the keys leaves a partial sum per query head, and all heads share the one kv head: the
+            # slices are counted as for a quarter of the heads as kv heads (measured at 16 heads: the kernel library's
+            # count for one kv head costs half as much again at 8,000 keys, and twice as much at 64 sequences)
+            keys = ctx.max_rows_visible(site)
             out = ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, rows_cap, self.scale, 0.0, 0,
-                                       ctx.dtype, max_keys=ctx.max_rows_visible(site))
+                                       ctx.dtype, max_keys=keys, splits=ops.decode_splits(m * max(1, H // 4), 1, row, keys))
         else:
             if owns:
                 ctx.offer_step_rows(latent=mine)
