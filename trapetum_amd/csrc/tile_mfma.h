@@ -5,7 +5,8 @@
 // the 64 up rows of the same units, and every lane ends up with a unit's gate and up sum in accumulators of the same
 // index; or the two sets are 128 neighbouring columns of a plain product.
 // K is walked in steps of 64 through one LDS buffer; the pieces of the step DEPTH steps ahead are asked for before the
-// current step is multiplied and written to LDS when their turn comes (few rows stream W: two steps in flight then).  The callers supply the loads: la8(m, k) and lw8(n, k) return the 8
+// current step is multiplied and written to LDS when their turn comes (few rows stream W: four steps in flight then;
+// an expert's products of a decode step: 161 -> 139 us against one step).  The callers supply the loads: la8(m, k) and lw8(n, k) return the 8
 // elements from k on of the tile's row m of A and row n of W (n < 128 when GATED: 64 gate rows, then 64 up rows),
 // zeros outside the operand.
 #pragma once
@@ -22,7 +23,7 @@ template <int TM, bool GATED>
 struct MfmaTile {
     static constexpr int WN = GATED ? 128 : 64;
     static constexpr int MI = TM >= 64 ? TM / 32 : 1, NJ = TM >= 64 ? 2 : 1, SETS = GATED ? 2 : 1;
-    static constexpr int DEPTH = TM >= 64 ? 1 : 2;
+    static constexpr int DEPTH = TM >= 64 ? 1 : 4;
     static constexpr int A_PIECES = TM * 8 / 256 > 0 ? TM * 8 / 256 : 1, W_PIECES = WN * 8 / 256;
     struct Shared { alignas(16) bf16_t a[TM][TMF_ROW]; alignas(16) bf16_t w[WN][TMF_ROW]; };
     tm_f32x4 acc[SETS][MI][NJ];
