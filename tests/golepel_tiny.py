@@ -35,6 +35,7 @@ def _moe(ff, limit, experts, top):
 def config_p(scale=1.0):
     a = dict(heads=3, dim=16, rot_dim=16, vdim=24, kv_rank=32, scale=0.2 * scale, base=500.0, dims=8)
     b = dict(heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=24, scale=0.3 * scale, base=77.0, dims=8)
+    c = dict(a, heads=5, dim=8, vdim=12, scale=0.25 * scale)       # reads a's cache with other heads, sizes and scale
     L = lambda m, mlp: {"type": "latent_attention", "mixer": m, "mlp": mlp}
     return {"architecture": "Golepel", "vocab": 211, "width": 96, "logit_scale": 0.7,
             "norm": {"eps": 1e-5, "groups": 3}, "canon": {"taps": 4},
@@ -42,7 +43,7 @@ def config_p(scale=1.0):
                        L(_mixer(**a, kv_from=0), {"kind": "dense", "ff": 72}),
                        L(_mixer(**b), None),
                        L(_mixer(**b, kv_from=2), _moe(24, 1.1, 4, 1)),
-                       L(_mixer(**a, kv_from=0), {"kind": "dense", "ff": 56})]}
+                       L(_mixer(**c, kv_from=0), {"kind": "dense", "ff": 56})]}
 
 
 def config_q():

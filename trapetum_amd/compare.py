@@ -59,12 +59,9 @@ class Run:
         self.sampler = Sampler(self.model.rt, SamplingParams())
         self.gen = torch.Generator().manual_seed(2)
         torch.cuda.synchronize()
-        self.weight_bytes = sum(t.numel() * 2 for t in self._tensors())
-        print(f"[compare] {name} ready in {time.time() - t0:.1f}s, {self.weight_bytes / 1e9:.2f} GB of weights", file=sys.stderr, flush=True)
-
-    def _tensors(self):
         import math
-        return [type("T", (), {"numel": lambda self, s=ts.shape: math.prod(s)})() for ts in self.model.tensor_layout().values()]
+        self.weight_bytes = 2 * sum(math.prod(ts.shape) for ts in self.model.tensor_layout().values())
+        print(f"[compare] {name} ready in {time.time() - t0:.1f}s, {self.weight_bytes / 1e9:.2f} GB of weights", file=sys.stderr, flush=True)
 
     def prompts(self, lengths):
         import torch
