@@ -160,11 +160,12 @@ def test_head_linear(rt, m, h, n, k, lead):
     assert bool((wide[:, :, :lead] == 7.0).all())
 
 
+@pytest.mark.parametrize("H", [4, 24])              # 24: more heads than a decode launch takes, run in groups
 @pytest.mark.parametrize("page,counts", [(16, (15, 1, 1, 1, 31, 2, 1, 40, 1, 1, 1, 1, 1, 2)), (64, (64, 1, 30, 1, 1, 1, 1, 1))])
-def test_latent_attention_sharp_scores(rt, page, counts):
+def test_latent_attention_sharp_scores(rt, page, counts, H):
     """Scores scaled until a softmax picks single keys, wherever they lie: a key lost or read one row off, at a page's
     border or far back, then changes a row's output by about as much as the output itself."""
-    H, dn, dr, dv, R, rot = 4, 16, 16, 16, 48, 16
+    dn, dr, dv, R, rot = 16, 16, 16, 48, 16
     part, W, sizes = latent_part(rt, H, dn, dr, dv, R, rot, scale=2.5)
     n = sum(counts)
     x_dev, x = acts(rt, rnd(n, 72, seed=10))

@@ -498,8 +498,18 @@ class HipOps:
         return self._linear(x, w_packed, out_dtype, EPI_GATED, 0.0, inter, act=GATE_ACTIVATIONS[activation])
 
     # ---- attention -------------------------------------------------------------------------------------
-    def _fast_attention(self, dtype, H, KV, hd):
-        return not self.force_plain_attention and dtype == torch.bfloat16 and hd % 16 == 0 and hd <= 256 and H // KV <= 16
+    DECODE_GROUP = 16              # query heads per kv head the matrix-core decode kernel takes
+
+    def _fast_attention(self, dtype, H, KV, hd, decode=True):
+        """Whether the matrix-core kernels take this geometry; the kernel of many queries takes any number of query
+        heads per kv head, the decode kernel up to DECODE_GROUP."""
+        return not self.force_plain_attention and dtype == torch.bfloat16 and hd % 16 == 0 and hd <= 256 and \
+            (not decode or H // KV <= self.DECODE_GROUP)
+
+    def decode_group_limit(self, dtype, hd):
+        """The most query heads per kv head a decode step's matrix-core attention takes in one call (a mixer whose
+        heads all share one kv head calls it for groups of them), or 0 where that kernel does not apply."""
+        return self.DECODE_GROUP if self._fast_attention(dtype, 1, 1, hd) else 0
 
     def attention_prefill(self, q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype,
                           row_seq=None, row_pos=None, cached=None, shape=0):
@@ -525,7 +535,7 @@ class HipOps:
             page, table_w, rows_cap = k_pool.shape[2], table.shape[1], rows_cap or 0
         ptr = lambda t: t.data_ptr() if t is not None else None
         out = torch.empty((m, H * hd), dtype=out_dtype, device=self.device)
-        if self._fast_attention(q.dtype, H, KV, hd) and (cached is None or (page >= 16 and page & (page - 1) == 0)):
+        if self._fast_attention(q.dtype, H, KV, hd, decode=False) and (cached is None or (page >= 16 and page & (page - 1) == 0)):
             lib = self.attn_lib(hd)
             self._call(lib, "tp_attn_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs,
                        m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count), ptr(new_len), ptr(table), table_w,

@@ -99,6 +99,20 @@ class LatentAttention(Mixer):
             # slices are counted as for a quarter of the heads as kv heads (measured at 16 heads: the kernel library's
             # count for one kv head costs half as much again at 8,000 keys, and twice as much at 64 sequences)
             keys = ctx.max_rows_visible(site)
+            limit = ops.decode_group_limit(ctx.dtype, row)
+            if limit and H > limit:
+                # more heads on the one kv head than the decode kernel takes: it runs for groups of them, each group's
+                # weighted latents going through its heads' W_uv into their place
+                heads = None
+                for h0 in range(0, H, limit):
+                    hg = min(limit, H - h0)
+                    part = ops.attention_decode(q[:, h0 * row:(h0 + hg) * row], hg, 1, row, ctx.new_len, table, pool, pool, rows_cap,
+                                                self.scale, 0.0, 0, ctx.dtype, max_keys=keys,
+                                                splits=ops.decode_splits(m * max(1, hg // 4), 1, row, keys))
+                    if heads is None:
+                        heads = part.new_empty((m, H, dv))
+                    ops.head_linear(part.view(m, hg, row)[:, :, dr:], self.w_up[h0:h0 + hg], heads[:, h0:h0 + hg])
+                return ops.linear(heads.view(m, H * dv), self.w_o, ctx.dtype, defer=True)
             out = ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, rows_cap, self.scale, 0.0, 0,
                                        ctx.dtype, max_keys=keys, splits=ops.decode_splits(m * max(1, H // 4), 1, row, keys))
         else:
