@@ -43,12 +43,16 @@ def test_schedules_agree(folder):
 
 
 def test_cache_is_sized_by_max_tokens(folder):
-    requests = {"a": list(range(65)), "b": list(range(10))}
-    steps = ts.batches(requests, 2, prefill_fraction=1.0)
-    assert ts.held_tokens(steps) == 128 + 64
+    """--max-tokens counts tokens, not pages: requests whose last pages are partly empty fit when the number is the
+    plain sum of their lengths, and what goes far beyond it is refused."""
+    from trapetum_amd.engine.trace import PAGE, SPARE_REQUESTS
+    requests = {"a": list(range(65)), "b": list(range(10)), "c": list(range(65))}
+    steps = ts.batches(requests, 3, prefill_fraction=1.0)
+    assert ts.held_tokens(steps) == 128 + 64 + 128
+    run(folder, steps, 65 + 10 + 65)
+    r = TraceRunner(folder, "float32", 140, device="cpu", ops=ref_ops_namespace())
     with pytest.raises(CacheError):
-        run(folder, steps, 128)
-    run(folder, steps, 192)
+        r.run_step({"step": 0, "entries": [{"id": "a", "tokens": [1] * (140 + SPARE_REQUESTS * PAGE + 1), "want": []}], "end": []})
 
 
 def test_steps_of_any_shape_and_what_is_still_refused(folder):
@@ -65,8 +69,8 @@ def test_steps_of_any_shape_and_what_is_still_refused(folder):
     with pytest.raises(StepError):       # a token outside the vocabulary; the newcomer's slot is given back
         r.run_step({"step": 3, "entries": [{"id": "a", "tokens": [7], "want": []}, {"id": "c", "tokens": [100000], "want": []}], "end": []})
     assert "c" not in r.slot_of and r.cache.length(r.slot_of["a"]) == 6
-    with pytest.raises(CacheError):      # more tokens than the cache was sized for
-        r.run_step({"step": 3, "entries": [{"id": "a", "tokens": list(range(200)), "want": []}], "end": []})
+    with pytest.raises(CacheError):      # far more tokens than the cache was sized for
+        r.run_step({"step": 3, "entries": [{"id": "a", "tokens": [1] * 20000, "want": []}], "end": []})
     assert r.cache.length(r.slot_of["a"]) == 6
     with pytest.raises(TraceError):
         r.run_step({"step": 4, "entries": [], "end": ["zz"]})

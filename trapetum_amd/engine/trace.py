@@ -23,6 +23,9 @@ from .model import Model
 from .runtime import Runtime
 
 PAGE = 64
+# Room beyond --max-tokens: that number counts the tokens live requests hold, and every live request's last page is
+# partly empty; pages for that many requests' last pages are added, so that the number need not be rounded by the caller.
+SPARE_REQUESTS = 256
 
 
 class TraceError(ValueError):
@@ -34,7 +37,8 @@ class TraceRunner:
         arch, self.config = config_from_folder(folder)
         self.model = Model(arch.build_spec(self.config), Runtime(dtype=dtype, device=device, ops=ops))
         load_folder(self.model, folder)
-        self.cache = self.model.new_cache(max_tokens, max_context=max_tokens, page_size=PAGE)
+        room = max(1, int(max_tokens)) + SPARE_REQUESTS * PAGE
+        self.cache = self.model.new_cache(room, max_context=room, max_slots=max(SPARE_REQUESTS, -(-room // PAGE)), page_size=PAGE)
         self.slot_of = {}
 
     def run_step(self, record):
@@ -83,7 +87,7 @@ def main(argv=None, stdin=None, stdout=None):
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder the logits files go to")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time, each rounded up to a multiple of 64")
+                    help="most tokens live requests hold at any time (a partly filled last page per request comes on top)")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
     stdin = stdin or sys.stdin
