@@ -212,6 +212,71 @@ expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
         }
 }
 
+// The same for the few pairs of a decode step, where the experts' matrices are streamed once and nothing is reused:
+// no LDS and no barrier.  A block takes 16 pairs of one expert x 64 columns, a wave 16 of the columns (GATED: the gate
+// and the up rows of 16 units); a lane reads its row of W and its pair's row of A straight into the matrix
+// instruction's operands, UN k steps of 32 asked for at once, so that a wave alone keeps a dozen kilobytes in flight.
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+expert_stream_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
+                int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out, int k_slice, long out_slice) {
+    constexpr int TM = 16, UN = 8;
+    int t = blockIdx.y, e = 0, lo = 0, hi = 0;
+    for (; e < E; e++) {
+        lo = first[e]; hi = first[e + 1];
+        const int tiles = (hi - lo + TM - 1) / TM;
+        if (t < tiles) break;
+        t -= tiles;
+    }
+    if (e == E) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+    const int p0 = lo + t * TM, n0 = blockIdx.x * 64 + wave * 16;
+    if (n0 >= N) return;
+    const int kz = blockIdx.z * k_slice, klen = min(K - kz, k_slice);
+    const int p = p0 + r, nw = n0 + r;
+    const bool a_ok = p < hi, w_ok = nw < N;
+    const size_t arow = a_ok ? (size_t)(GATED ? order[p] / top : p) : 0;
+    const bf16_t* ap = a + arow * K + kz + g * 8;
+    const bf16_t* we = w + (size_t)e * (GATED ? 2 : 1) * N * K;
+    const bf16_t* wg = we + (size_t)(w_ok ? nw : 0) * K + kz + g * 8;
+    const bf16_t* wu = wg + (size_t)N * K;               // the unit's up row (gated)
+    tm_f32x4 acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    union F { uint4 u; tm_bf16x8 v; };
+    for (int k0 = 0; k0 < klen; k0 += 32 * UN) {
+        F fa[UN], fg[UN], fu[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int k = k0 + 32 * u;
+            const bool in = k + g * 8 < klen;
+            fa[u].u = (in && a_ok) ? *reinterpret_cast<const uint4*>(ap + k) : zero;
+            fg[u].u = (in && w_ok) ? *reinterpret_cast<const uint4*>(wg + k) : zero;
+            if (GATED) fu[u].u = (in && w_ok) ? *reinterpret_cast<const uint4*>(wu + k) : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg[u].v, fa[u].v, acc_g, 0, 0, 0);
+            if (GATED) acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu[u].v, fa[u].v, acc_u, 0, 0, 0);
+        }
+    }
+    // the lane holds pair r, columns n0 + g * 4 + v
+    if (!a_ok) return;
+    const int n = n0 + g * 4;
+    if constexpr (GATED) {
+        bf16_t* dst = (bf16_t*)out + (size_t)p * N + n;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            if (n + v >= N) continue;
+            const float gg = fminf(acc_g[v], limit), uu = fminf(fmaxf(acc_u[v], -limit), limit);
+            dst[v] = f32_to_bf16(gg / (1.f + expf(-alpha * gg)) * (uu + shift));
+        }
+    } else {
+        float* dst = (float*)out + (size_t)blockIdx.z * out_slice + (size_t)p * N + n;
+#pragma unroll
+        for (int v = 0; v < 4; v++) if (n + v < N) dst[v] = acc_g[v];
+    }
+}
+
 // ---- out[m] = sum_k weight[m, k] * pair_out[place[m top + k]], k ascending, float32.  grid (rows, column blocks) ------
 // K slices the down product of a decode step is cut in (when the experts' width allows slices of whole steps)
 static int down_slices(int P, int F) { return (P <= 64 && F >= 1024 && F % 256 == 0) ? 4 : 1; }
@@ -267,10 +332,14 @@ extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* 
 #define TP_EXPERT_MFMA(G, TMv, Nv, Kv, A, W, O, Z) expert_linear_mfma_k<G, TMv><<<dim3(tp_cdiv(Nv, (G) == 2 ? 128 : 64), row_tiles, Z), 256, 0, s>>>( \
         (const bf16_t*)(A), (const bf16_t*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O, (Kv) / (Z), (long)P * (Nv))
     if (cores) {
-        if (few) TP_EXPERT_MFMA(1, 16, F, D, x, w_gate_up, y, 1); else if (many) TP_EXPERT_MFMA(1, 128, F, D, x, w_gate_up, y, 1); else TP_EXPERT_MFMA(1, 64, F, D, x, w_gate_up, y, 1);
+        if (few) expert_stream_k<true><<<dim3(tp_cdiv(F, 64), row_tiles, 1), 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w_gate_up, order, first, E, top, F, D,
+                                                                                             limit, alpha, shift, y, D, 0);
+        else if (many) TP_EXPERT_MFMA(1, 128, F, D, x, w_gate_up, y, 1); else TP_EXPERT_MFMA(1, 64, F, D, x, w_gate_up, y, 1);
         if (int rc = tp_check_launch("expert_ffn (gate, up; matrix cores)")) return rc;
         const int zs = down_slices(P, F);
-        if (few) TP_EXPERT_MFMA(0, 16, D, F, y, w_down, pair_out, zs); else if (many) TP_EXPERT_MFMA(2, 128, D, F, y, w_down, pair_out, 1); else TP_EXPERT_MFMA(0, 64, D, F, y, w_down, pair_out, 1);
+        if (few) expert_stream_k<false><<<dim3(tp_cdiv(D, 64), row_tiles, zs), 256, 0, s>>>((const bf16_t*)y, (const bf16_t*)w_down, order, first, E, top, D, F,
+                                                                                               limit, alpha, shift, pair_out, F / zs, (long)P * D);
+        else if (many) TP_EXPERT_MFMA(2, 128, D, F, y, w_down, pair_out, 1); else TP_EXPERT_MFMA(0, 64, D, F, y, w_down, pair_out, 1);
         if (int rc = tp_check_launch("expert_ffn (down; matrix cores)")) return rc;
         expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, zs, (long)P * D, place, weight, top, D, out);
         return tp_check_launch("expert_ffn (combine)");

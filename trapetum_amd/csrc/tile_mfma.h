@@ -5,8 +5,7 @@
 // the 64 up rows of the same units, and every lane ends up with a unit's gate and up sum in accumulators of the same
 // index; or the two sets are 128 neighbouring columns of a plain product.
 // K is walked in steps of 64 through one LDS buffer; the pieces of the step DEPTH steps ahead are asked for before the
-// current step is multiplied and written to LDS when their turn comes (few rows stream W: four steps in flight then;
-// an expert's products of a decode step: 161 -> 139 us against one step).  The callers supply the loads: la8(m, k) and lw8(n, k) return the 8
+// current step is multiplied and written to LDS when their turn comes (few rows stream W: four steps in flight then).  The callers supply the loads: la8(m, k) and lw8(n, k) return the 8
 // elements from k on of the tile's row m of A and row n of W (n < 128 when GATED: 64 gate rows, then 64 up rows),
 // zeros outside the operand.
 #pragma once
