@@ -190,7 +190,8 @@ def test_latent_attention_sharp_scores(rt, page, counts, H):
 
 
 @pytest.mark.parametrize("m,d,f,e,top,limit", [(1, 64, 40, 5, 3, 0.8), (9, 50, 18, 2, 2, 0.5), (150, 96, 70, 16, 2, 1.5),
-                                               (70, 128, 33, 9, 1, 2.0), (300, 72, 24, 130, 4, 1.0), (650, 136, 200, 3, 2, 1.2), (5, 64, 1024, 3, 2, 1.0)])
+                                               (70, 128, 33, 9, 1, 2.0), (300, 72, 24, 130, 4, 1.0), (650, 136, 200, 3, 2, 1.2), (5, 64, 1024, 3, 2, 1.0),
+                                               (700, 128, 192, 3, 2, 1.0), (530, 192, 320, 2, 2, 0.9), (900, 64, 64, 7, 1, 1.5)])
 def test_routed_experts(rt, m, d, f, e, top, limit):
     part = build_part("feed_forward", ("routed_experts", dict(hidden_size=d, intermediate_size=f, n_experts=e, top=top, limit=limit)))
     dev, W = {}, {}

@@ -212,6 +212,140 @@ expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
         }
 }
 
+// The products of many pairs (a prefill) when K is whole steps of 64: tiles of 128 pairs x 128 rows of W (GATED: 64 units'
+// gate rows and up rows; else 128 columns), the step's tile straight from global memory into LDS
+// (global_load_lds_dwordx4: no staging registers, no LDS writes), as the dense products' loop does it: a step reads all
+// its fragments into registers, a barrier, the next step's loads are issued into the same buffer and fly while the
+// step's 32 matrix instructions run, a second barrier when they have landed.  A lane's place in LDS is fixed by its
+// lane number, so the swizzle (piece ^ (row & 7)) is applied on the global side; a row of A is the pair's token row
+// (gathered through `order`), rows past a run's end or past N fetch a row that exists and are never stored.
+template <bool GATED>
+__global__ void __launch_bounds__(256, 2)
+expert_direct_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
+                int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out) {
+    constexpr int BM = 128, BN = 128, BK = 64, LDS = BK, TM = 4, TN = 4;
+    __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
+    __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
+    int t = blockIdx.y, e = 0, lo = 0, hi = 0;
+    for (; e < E; e++) {
+        lo = first[e]; hi = first[e + 1];
+        const int tiles = (hi - lo + BM - 1) / BM;
+        if (t < tiles) break;
+        t -= tiles;
+    }
+    if (e == E) return;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int p0 = lo + t * BM, n0 = blockIdx.x * (GATED ? 64 : 128);
+    const bf16_t* we = w + (size_t)e * (GATED ? 2 : 1) * N * K;
+    // load i of a thread: row (tid >> 3) + 32 i of the tile, the piece that belongs at the lane's place
+    const int srow = tid >> 3, chunk = (lane & 7) ^ (srow & 7);
+    unsigned xo[TM], wo[TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int p = min(p0 + srow + 32 * i, hi - 1);
+        const int row = GATED ? order[p] / top : p;
+        xo[i] = (unsigned)row * (unsigned)K * 2u + chunk * 16u;
+    }
+#pragma unroll
+    for (int i = 0; i < TN; i++) {
+        const int sr = srow + 32 * i;                    // staged row of W: gated 0 .. 63 gate, 64 .. 127 up of the same units
+        const int wrow = GATED ? (sr >= 64 ? N : 0) + min(n0 + (sr & 63), N - 1) : min(n0 + sr, N - 1);
+        wo[i] = (unsigned)wrow * (unsigned)K * 2u + chunk * 16u;
+    }
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    bf16_t* const a_dst = As + wave_u * 8 * LDS;         // the wave's 8 rows of every group of 32
+    bf16_t* const b_dst = Bs + wave_u * 8 * LDS;
+    auto fill = [&](int k0) {
+        const char* xb = reinterpret_cast<const char*>(a) + (size_t)k0 * 2;
+        const char* wb = reinterpret_cast<const char*>(we) + (size_t)k0 * 2;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + xo[i]),
+                                             (__attribute__((address_space(3))) void*)(a_dst + 32 * i * LDS), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wb + wo[i]),
+                                             (__attribute__((address_space(3))) void*)(b_dst + 32 * i * LDS), 16, 0, 0);
+    };
+    union Frag { uint4 u; tm_bf16x8 v; };
+    tm_f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = tm_f32x4{0.f, 0.f, 0.f, 0.f};
+    // the wave's rows of W in the staged tile: gated, accumulators j and j + 2 are a unit's gate and up sums
+    auto w_row = [&](int j) { return GATED ? (j >= 2 ? 64 : 0) + wn * 32 + (j & 1) * 16 : wn * 64 + j * 16; };
+    auto frags = [&](int ks, Frag (&fa)[TM], Frag (&fb)[TN]) {
+        const int kc = (((ks >> 3) + g) ^ (r & 7)) * 8;
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[i].u = *reinterpret_cast<const uint4*>(As + (wm * 64 + i * 16 + r) * LDS + kc);
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[j].u = *reinterpret_cast<const uint4*>(Bs + (w_row(j) + r) * LDS + kc);
+    };
+    auto mma = [&](Frag (&fa)[TM], Frag (&fb)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j].v, fa[i].v, acc[i][j], 0, 0, 0);
+    };
+    fill(0);
+    __builtin_amdgcn_s_waitcnt(0);                       // every counter at zero: the loads have reached LDS
+    __syncthreads();
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        Frag a0[TM], b0[TN], a1[TM], b1[TN];
+        frags(0, a0, b0);
+        frags(32, a1, b1);
+        __builtin_amdgcn_s_waitcnt(0);                   // the fragments are in registers ...
+        __syncthreads();                                 // ... everyone's: the buffer may be refilled
+        if (k0 + BK < K) fill(k0 + BK);
+        mma(a0, b0);
+        mma(a1, b1);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
+    // the lane holds pair row wm * 64 + i * 16 + r, rows of W w_row(j) + g * 4 + v
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int p = p0 + wm * 64 + i * 16 + r;
+        if (p >= hi) continue;
+        if constexpr (GATED) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int n = n0 + wn * 32 + j * 16 + g * 4;
+                bf16_t o[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float gg = fminf(acc[i][j][v], limit), uu = fminf(fmaxf(acc[i][j + 2][v], -limit), limit);
+                    o[v] = f32_to_bf16(gg / (1.f + expf(-alpha * gg)) * (uu + shift));
+                }
+                bf16_t* dst = (bf16_t*)out + (size_t)p * N + n;
+                if ((N & 3) == 0 && n + 3 < N) {
+                    uint2 pk;
+                    pk.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+                    pk.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+                    *reinterpret_cast<uint2*>(dst) = pk;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) if (n + v < N) dst[v] = o[v];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int n = n0 + wn * 64 + j * 16 + g * 4;
+                float* dst = (float*)out + (size_t)p * N + n;
+                if ((N & 3) == 0 && n + 3 < N) *reinterpret_cast<float4*>(dst) = make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+                else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) if (n + v < N) dst[v] = acc[i][j][v];
+                }
+            }
+        }
+    }
+}
+
 // The same for the few pairs of a decode step, where the experts' matrices are streamed once and nothing is reused:
 // no LDS and no barrier.  A block takes 16 pairs of one expert x 64 columns, a wave 16 of the columns (GATED: the gate
 // and the up rows of 16 units); a lane reads its row of W and its pair's row of A straight into the matrix
@@ -334,11 +468,17 @@ extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* 
     if (cores) {
         if (few) expert_stream_k<true><<<dim3(tp_cdiv(F, 64), row_tiles, 1), 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w_gate_up, order, first, E, top, F, D,
                                                                                              limit, alpha, shift, y, D, 0);
+        else if (many && D % 64 == 0 && (long)M * D * 2 < (1L << 32) && 2L * F * D * 2 < (1L << 32))
+            expert_direct_k<true><<<dim3(tp_cdiv(F, 64), row_tiles), 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w_gate_up, order, first, E, top, F, D,
+                                                                                  limit, alpha, shift, y);
         else if (many) TP_EXPERT_MFMA(1, 128, F, D, x, w_gate_up, y, 1); else TP_EXPERT_MFMA(1, 64, F, D, x, w_gate_up, y, 1);
         if (int rc = tp_check_launch("expert_ffn (gate, up; matrix cores)")) return rc;
         const int zs = down_slices(P, F);
         if (few) expert_stream_k<false><<<dim3(tp_cdiv(D, 64), row_tiles, zs), 256, 0, s>>>((const bf16_t*)y, (const bf16_t*)w_down, order, first, E, top, D, F,
                                                                                                limit, alpha, shift, pair_out, F / zs, (long)P * D);
+        else if (many && F % 64 == 0 && (long)P * F * 2 < (1L << 32) && (long)D * F * 2 < (1L << 32))
+            expert_direct_k<false><<<dim3(tp_cdiv(D, 128), row_tiles), 256, 0, s>>>((const bf16_t*)y, (const bf16_t*)w_down, order, first, E, top, D, F,
+                                                                                    limit, alpha, shift, pair_out);
         else if (many) TP_EXPERT_MFMA(2, 128, D, F, y, w_down, pair_out, 1); else TP_EXPERT_MFMA(0, 64, D, F, y, w_down, pair_out, 1);
         if (int rc = tp_check_launch("expert_ffn (down; matrix cores)")) return rc;
         expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, zs, (long)P * D, place, weight, top, D, out);
