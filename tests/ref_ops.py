@@ -229,11 +229,7 @@ def decode_splits(n, KV, hd, keys):
     return 1
 
 
-def decode_group_limit(dtype, hd):
-    return 0
-
-
-def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype, max_keys=None, splits=None):
+def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype, max_keys=None, splits=None, head_groups=None):
     n = q.shape[0]
     page = k_pool.shape[2]
     out = torch.zeros((n, H * hd), dtype=torch.float32, device=q.device)

@@ -187,7 +187,10 @@ def time_golepel_kernels(engine, cfg, batch, context, prefill_tokens):
             one([(lambda b=b: ops.head_linear(xq, b.mixer.w_absorb, qv)) for b in blocks], name="absorb",
                 bytes_each=2.0 * (elems(mx.w_absorb) + rows * H * (dn + R)))
             if decode:
-                one([lambda: ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, 0, mx.scale, 0.0, 0, bf, max_keys=context)] * 8,
+                # as the mixer calls it: the heads in groups that each read the shared cached rows
+                per = next(g for g in (mx.DECODE_GROUP_LONG if context >= mx.LONG_KEYS else mx.DECODE_GROUP, 4, 2, 1) if H % g == 0)
+                one([lambda: ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, 0, mx.scale, 0.0, 0, bf, max_keys=context,
+                                                  head_groups=H // per, splits=ops.decode_splits(batch * (H // per), 1, row, context))] * 8,
                     name=f"attention_ctx{context}", bytes_each=2.0 * batch * context * row)
             else:
                 pairs = rows * (rows + 1) / 2.0

@@ -70,6 +70,9 @@ struct DecodeArgs {
     // [heads | kv heads (keys) | kv heads (values)] x head size, bf16, or float32 in K slices that are added here
     const void* qkv; int qkv_f32, n_slices; long slice_stride, row_stride;
     const float* inv_freq; int rot, write_kv;
+    // kv heads the pools really have (0: KV).  Fewer than KV: the grid's kv heads are groups of query heads that share
+    // pool head `kvh % pool_kv` (a cache with one row per token for all heads is read by every group)
+    int pool_kv;
 };
 
 namespace {
@@ -122,7 +125,7 @@ attn_decode_k(DecodeArgs a) {
             row = row >= a.rows_cap ? row - a.rows_cap : row;
         }
         const int pg = table[row >> page_shift];
-        return (((size_t)pg * a.KV + kvh) * a.page + (row & page_mask)) * HD;
+        return (((size_t)pg * a.pool_kv + (a.pool_kv == a.KV ? kvh : kvh % a.pool_kv)) * a.page + (row & page_mask)) * HD;
     };
 
     // the lane's part in the weighted sum: chunk ch of the head, keys kgw, kgw + KGW, ... of the wave's 16
@@ -422,6 +425,9 @@ static int decode_launch(DecodeArgs a, int n_seq, void* workspace, hipStream_t s
     TP_REQUIRE(a.H % a.KV == 0, "attention: %d query heads are no multiple of %d kv heads", a.H, a.KV);
     const int G = a.H / a.KV;
     TP_REQUIRE(G <= 16, "attention decode (matrix-core kernel): %d query heads per kv head exceed 16", G);
+    if (a.pool_kv == 0) a.pool_kv = a.KV;
+    TP_REQUIRE(a.pool_kv > 0 && a.KV % a.pool_kv == 0 && (a.pool_kv == a.KV || !a.qkv),
+               "attention decode: %d groups of heads cannot share %d kv heads of the cache", a.KV, a.pool_kv);
     TP_REQUIRE(a.page >= 16 && (a.page & (a.page - 1)) == 0 && a.table_w > 0, "attention decode (matrix-core kernel): page size %d must be a power of two, at least 16", a.page);
     TP_REQUIRE(a.rows_cap == 0 || a.window <= a.rows_cap, "attention decode: a window of %d keys does not fit a ring of %d rows", a.window, a.rows_cap);
     TP_REQUIRE(a.rows_cap >= 0 && a.rows_cap % a.page == 0, "attention decode: ring of %d rows is no multiple of the page size %d", a.rows_cap, a.page);
@@ -453,6 +459,20 @@ extern "C" int tp_attn_decode(const void* q, long q_stride, int n_seq, int H, in
     DecodeArgs a{(const bf16_t*)q, q_stride, H, KV, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool,
                  page, rows_cap, scale, cap, window, (bf16_t*)out, nullptr, nullptr, nsplit,
                  nullptr, 0, 1, 0, 0, nullptr, 0, 0};
+    return decode_launch(a, n_seq, workspace, (hipStream_t)stream);
+}
+
+// The same over a cache with `pool_kv` kv heads read by `KV` groups of query heads (KV a multiple of pool_kv): group j
+// reads pool head j % pool_kv.  With one row per token for all heads (pool_kv 1) the heads are cut into groups, each a
+// block's worth of weighted sums, instead of one block forming all of them.
+extern "C" int tp_attn_decode_shared(const void* q, long q_stride, int n_seq, int H, int KV, int pool_kv, const int* new_len,
+                                     const int* table, int table_w, const void* k_pool, const void* v_pool, int page,
+                                     int rows_cap, float scale, float cap, int window, void* out, void* workspace,
+                                     int nsplit, void* stream) {
+    TP_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "attention decode: query rows must be 16-byte aligned");
+    DecodeArgs a{(const bf16_t*)q, q_stride, H, KV, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool,
+                 page, rows_cap, scale, cap, window, (bf16_t*)out, nullptr, nullptr, nsplit,
+                 nullptr, 0, 1, 0, 0, nullptr, 0, 0, pool_kv};
     return decode_launch(a, n_seq, workspace, (hipStream_t)stream);
 }
 

@@ -46,6 +46,7 @@ _CORE_SIGS = {
 _ATTN_SIGS = {
     "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _I, _P],
     "tp_attn_decode": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
+    "tp_attn_decode_shared": [_P, _L, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
     "tp_attn_decode_workspace_floats": [_I, _I, _I],
     "tp_attn_decode_fused": [_P, _I, _I, _L, _L, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
 }
@@ -506,11 +507,6 @@ class HipOps:
         return not self.force_plain_attention and dtype == torch.bfloat16 and hd % 16 == 0 and hd <= 256 and \
             (not decode or H // KV <= self.DECODE_GROUP)
 
-    def decode_group_limit(self, dtype, hd):
-        """The most query heads per kv head a decode step's matrix-core attention takes in one call (a mixer whose
-        heads all share one kv head calls it for groups of them), or 0 where that kernel does not apply."""
-        return self.DECODE_GROUP if self._fast_attention(dtype, 1, 1, hd) else 0
-
     def attention_prefill(self, q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype,
                           row_seq=None, row_pos=None, cached=None, shape=0):
         """Causal attention of the step's queries over the step's own rows of keys and values and, with
@@ -574,7 +570,10 @@ class HipOps:
             raise KernelError(f"{what}: the page table must be contiguous int32 [sequences, pages]")
 
     def attention_decode(self, q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window,
-                         out_dtype, max_keys=None, splits=None):
+                         out_dtype, max_keys=None, splits=None, head_groups=None):
+        """head_groups: cut the query heads into that many groups (a multiple of KV), each read the pool head
+        `group % KV` by a block of its own: for caches whose one kv head serves many heads, where one block would
+        otherwise form all their weighted sums.  The plain kernel takes any grouping as it is."""
         self._dev(q, new_len, table, k_pool, v_pool)
         n = q.shape[0]
         qs = self._rows(q, "attention q")
@@ -583,12 +582,21 @@ class HipOps:
         self._check_pools("attention_decode", q.dtype, n, KV, hd, new_len, table, k_pool, v_pool)
         out = torch.empty((n, H * hd), dtype=out_dtype, device=self.device)
         page = k_pool.shape[2]
-        if self._fast_attention(q.dtype, H, KV, hd) and page >= 16 and page & (page - 1) == 0:
+        groups = int(head_groups) if head_groups else KV
+        if groups % KV or H % groups:
+            raise KernelError(f"attention_decode: {H} heads in {groups} groups on {KV} kv heads")
+        if self._fast_attention(q.dtype, H, groups, hd) and page >= 16 and page & (page - 1) == 0:
             lib = self.attn_lib(hd)
             keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
-            nsplit = int(splits) if splits else self.decode_splits(n, KV, hd, keys)
+            nsplit = int(splits) if splits else self.decode_splits(n, groups, hd, keys)
             floats = lib.tp_attn_decode_workspace_floats(n, H, nsplit)
             ws = torch.empty(floats, dtype=torch.float32, device=self.device) if floats else None
+            if groups != KV:
+                self._call(lib, "tp_attn_decode_shared", q.data_ptr(), qs, n, H, groups, KV, new_len.data_ptr(), table.data_ptr(),
+                           table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[2], rows_cap, float(scale),
+                           float(softcap), int(window), out.data_ptr(), ws.data_ptr() if ws is not None else None, nsplit,
+                           self._stream())
+                return out
             self._call(lib, "tp_attn_decode", q.data_ptr(), qs, n, H, KV, new_len.data_ptr(), table.data_ptr(),
                        table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[2], rows_cap, float(scale),
                        float(softcap), int(window), out.data_ptr(), ws.data_ptr() if ws is not None else None, nsplit,

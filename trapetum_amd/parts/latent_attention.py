@@ -22,6 +22,8 @@ from .base import Mixer
 
 
 class LatentAttention(Mixer):
+    DECODE_GROUP, DECODE_GROUP_LONG, LONG_KEYS = 4, 8, 1536       # query heads a block of the decode attention takes (see forward)
+
     def __init__(self, hidden_size, num_heads, nope_dim, rope_dim, value_dim, latent_rank, scale, latent_eps,
                  position=("none", {}), own_latent=True,
                  tensors=("q", "dkv", "dkv.norm", "uk", "uv", "o")):
@@ -95,26 +97,17 @@ class LatentAttention(Mixer):
                                      rows_cap, own=owns, out_dtype=ctx.dtype)
         ops.head_linear(proj[:, :H * (dr + dn)].view(m, H, dr + dn)[:, :, dr:], self.w_absorb, q.view(m, H, row)[:, :, dr:])
         if ctx.mode == "decode":
-            # every slice of the keys leaves a partial sum per query head, and all heads share the one kv head: the
-            # slices are counted as for a quarter of the heads as kv heads (measured at 16 heads: the kernel library's
-            # count for one kv head costs half as much again at 8,000 keys, and twice as much at 64 sequences)
+            # All heads share the one kv head.  A block of the decode kernel forms the weighted sums of a kv head's
+            # query heads by multiply-adds in its lanes, so the heads are cut into groups, each group a block of its
+            # own on the same cached rows, and the keys' slices are counted for that many kv heads.  Measured at 16
+            # heads and rows of 256 elements, heads a block 16 / 8 / 4 / 2: 8 sequences at 552 keys 18.3 / 13.4 / 11.9 /
+            # 11.2 us, at 2,048 keys 20.7 / 17.6 / 22.3 / 23.1, at 7,900 keys 68.7 / 39.6 / 46.2 / 51.9; 64 sequences at
+            # 552 keys 46.8 / 35.5 / 30.0 / 36.5.
             keys = ctx.max_rows_visible(site)
-            limit = ops.decode_group_limit(ctx.dtype, row)
-            if limit and H > limit:
-                # more heads on the one kv head than the decode kernel takes: it runs for groups of them, each group's
-                # weighted latents going through its heads' W_uv into their place
-                heads = None
-                for h0 in range(0, H, limit):
-                    hg = min(limit, H - h0)
-                    part = ops.attention_decode(q[:, h0 * row:(h0 + hg) * row], hg, 1, row, ctx.new_len, table, pool, pool, rows_cap,
-                                                self.scale, 0.0, 0, ctx.dtype, max_keys=keys,
-                                                splits=ops.decode_splits(m * max(1, hg // 4), 1, row, keys))
-                    if heads is None:
-                        heads = part.new_empty((m, H, dv))
-                    ops.head_linear(part.view(m, hg, row)[:, :, dr:], self.w_up[h0:h0 + hg], heads[:, h0:h0 + hg])
-                return ops.linear(heads.view(m, H * dv), self.w_o, ctx.dtype, defer=True)
+            per = next(g for g in (self.DECODE_GROUP_LONG if keys >= self.LONG_KEYS else self.DECODE_GROUP, 4, 2, 1) if H % g == 0)
             out = ops.attention_decode(q, H, 1, row, ctx.new_len, table, pool, pool, rows_cap, self.scale, 0.0, 0,
-                                       ctx.dtype, max_keys=keys, splits=ops.decode_splits(m * max(1, H // 4), 1, row, keys))
+                                       ctx.dtype, max_keys=keys, head_groups=H // per,
+                                       splits=ops.decode_splits(m * (H // per), 1, row, keys))
         else:
             if owns:
                 ctx.offer_step_rows(latent=mine)
