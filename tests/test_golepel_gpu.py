@@ -145,6 +145,33 @@ def test_latent_attention_part(rt, H, dn, dr, dv, R, rot):
     assert rel_l2(torch.cat(got2), want2) < tol
 
 
+def test_latent_attention_long_context(rt):
+    """Beyond 1,536 keys the decode attention takes the heads in groups of 8: a prompt of 1,600 tokens, then single tokens."""
+    H, dn, dr, dv, R, rot = 8, 16, 16, 16, 48, 16
+    part, W, sizes = latent_part(rt, H, dn, dr, dv, R, rot, scale=0.6)
+    n, first = 1640, 1600
+    x_dev, x = acts(rt, rnd(n, 72, seed=12))
+    pos = torch.arange(n)
+    lat = plain.latent_keys(x, W["mix.dkv"], W["mix.dkv.norm"], 1e-5, R, pos, sizes["rot"])
+    want = plain.latent_attention(x, W, "mix.", sizes, pos, lat)
+    cache = ModelCache([part.cache_spec()], 2048, 2048, 2, 64, rt.dtype, rt.device)
+    s = cache.acquire()
+    got, at = [], 0
+    for count in [first] + [1] * (n - first):
+        start = cache.length(s)
+        cache.grow(s, count)
+        ctx = StepContext(rt, cache, [s], [count], [start], [])
+        ctx.entry = ctx.cache_owner = 0
+        got.append(rt.ops.rows(part.forward(ctx, x_dev[at:at + count], cache.site(0)), rt.dtype))
+        at += count
+    got = torch.cat(got)
+    # float32 angles of a thousand radians and more are rounded to about 1e-4 of a radian: some 1e-5 of the output
+    tol = 5e-5 if rt.dtype == torch.float32 else 3e-2
+    assert rel_l2(got[:first], want[:first]) < tol
+    for i in range(first, n):
+        assert rel_l2(got[i], want[i]) < 2 * tol, i
+
+
 @pytest.mark.parametrize("m,h,n,k,lead", [(5, 3, 32, 16, 16), (100, 4, 24, 40, 8), (700, 2, 200, 72, 0), (9, 5, 7, 12, 6), (600, 3, 50, 24, 16)])
 def test_head_linear(rt, m, h, n, k, lead):
     """Per-head products on views of wider rows: each head's `k` elements follow `lead` others, and the output lands
