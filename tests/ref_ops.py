@@ -37,6 +37,8 @@ def rms_norm(x, gain, eps, out_dtype, groups=1):
 
 
 def add_rms_norm(stream, rows, gain_post, eps_post, gain_next, eps_next, out_dtype, groups=1):
+    if hasattr(rows, "slices"):
+        rows = rows.slices.sum(0)
     t = rows.float() if gain_post is None else _norm(rows, gain_post, eps_post, groups)
     stream += t
     if gain_next is None:
@@ -96,8 +98,8 @@ def head_linear(x, w, out=None):
     return out
 
 
-def route_top(logits, top, renormalize=False):
-    s = torch.softmax(logits.float(), dim=-1)
+def route_top(logits, top, renormalize=False, score="softmax"):
+    s = torch.softmax(logits.float(), dim=-1) if score == "softmax" else torch.sigmoid(logits.float())
     order = torch.argsort(-s, dim=-1, stable=True)[:, :top]
     w = torch.gather(s, 1, order)
     if renormalize:
@@ -105,27 +107,37 @@ def route_top(logits, top, renormalize=False):
     return order.to(torch.int32), w
 
 
-def expert_ffn(x, chosen, weights, w_gate_up, w_down, limit, alpha, shift):
-    """fp32 [M, D]: sum over a token's chosen experts, in the order they were chosen, of weight * expert(x)."""
+def expert_ffn(x, chosen, weights, w_gate_up, w_down, limit, alpha, shift, weight_input=False, out=None):
+    """fp32 [M, D]: sum over a token's chosen experts, in the order they were chosen, of weight * expert(x), or
+    (weight_input) of expert(weight * x): gate and up sums times the weight, before the clamps."""
     m, ff = x.shape[0], w_gate_up.shape[1] // 2
-    out = torch.zeros((m, w_down.shape[1]), dtype=torch.float32, device=x.device)
+    limit = float("inf") if limit is None else limit
+    res = torch.zeros((m, w_down.shape[1]), dtype=torch.float32, device=x.device)
     for k in range(chosen.shape[1]):
         for r in range(m):
             e = int(chosen[r, k])
             gu = w_gate_up[e].float() @ x[r].float()
+            if weight_input:
+                gu = gu * weights[r, k]
             g, u = torch.clamp(gu[:ff], max=limit), torch.clamp(gu[ff:], -limit, limit)
             y = (g * torch.sigmoid(alpha * g) * (u + shift)).to(x.dtype).float()
-            out[r] += weights[r, k] * (w_down[e].float() @ y)
+            res[r] += (1.0 if weight_input else weights[r, k]) * (w_down[e].float() @ y)
+    if out is None:
+        return res
+    out.copy_(res)
     return out
 
 
-def linear(x, w, out_dtype, softcap=None, defer=False, bias=None):
+def linear(x, w, out_dtype, softcap=None, defer=False, bias=None, out=None):
     y = x.float() @ w.float().T
     if bias is not None:
         y = y + bias.float()
     if softcap:
         y = softcap * torch.tanh(y / softcap)
-    return y.to(out_dtype)
+    if out is None:
+        return y.to(out_dtype)
+    out.copy_(y.to(out_dtype))
+    return out
 
 
 def _gelu_tanh(g):
@@ -133,7 +145,7 @@ def _gelu_tanh(g):
 
 
 def gated_linear(x, w_packed, inter, activation, out_dtype):
-    act = {"gelu_tanh": _gelu_tanh, "silu": lambda g: g * torch.sigmoid(g)}[activation]
+    act = {"gelu_tanh": _gelu_tanh, "silu": lambda g: g * torch.sigmoid(g), "relu": torch.relu}[activation]
     y = x.float() @ w_packed.float().T                     # [M, 2 * ip]
     y = y.reshape(x.shape[0], -1, 2, GROUP)
     g, u = y[:, :, 0, :].reshape(x.shape[0], -1), y[:, :, 1, :].reshape(x.shape[0], -1)
@@ -273,8 +285,69 @@ def attention_decode_step(qkv, H, KV, hd, inv_freq, rotary_dim, new_len, table, 
     return attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype)
 
 
+class SplitRows:
+    """The kernel library's rows in slices, fp32 [slices, M, N]: their sum is meant."""
+
+    def __init__(self, slices):
+        self.slices = slices
+        self.shape = tuple(slices.shape[1:])
+        self.dtype = torch.float32
+
+
 def rows(r, dtype):
+    if isinstance(r, SplitRows):
+        return r.slices.sum(0).to(dtype)
     return r
+
+
+def conv_act(x, w_t, bias, state, slot_ids, cu_rows, row_seq, activation=None, one_row_each=False):
+    """out_t = act(bias + sum_j w_t[j] x_(t - taps + 1 + j)); rows before the step come from state[slot] ([taps - 1, C],
+    oldest first), which then takes the last taps - 1 rows of (state, step)."""
+    taps = w_t.shape[0]
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    xf = x.float()
+    for i in range(len(cu_rows) - 1):
+        a, b, slot = int(cu_rows[i]), int(cu_rows[i + 1]), int(slot_ids[i])
+        hist = xf[a:b] if taps == 1 else torch.cat([state[slot], xf[a:b]])
+        acc = torch.zeros_like(xf[a:b]) if bias is None else bias.float().expand(b - a, -1).clone()
+        for j in range(taps):
+            acc += w_t[j] * hist[j:j + (b - a)]
+        out[a:b] = acc
+        if taps > 1:
+            state[slot] = hist[hist.shape[0] - (taps - 1):].clone()
+    if activation == "silu":
+        out = out * torch.sigmoid(out)
+    return out.to(x.dtype)
+
+
+def ssd_scan(xbc, z, dt, dt_bias, a_log, skip, state, slot_ids, cu_rows, max_count, heads, groups, n_state, head_dim):
+    """S <- exp(-exp(a_log) d) S + d B x^T, y = (S^T C + skip x) * silu(z), d = softplus(dt + dt_bias), row after row of
+    every sequence from state[slot] [heads, n_state, head_dim], which is left updated.  float32 [M, heads head_dim]."""
+    m, inner, gn = xbc.shape[0], heads * head_dim, groups * n_state
+    x = xbc[:, :inner].float().reshape(m, heads, head_dim)
+    B = xbc[:, inner:inner + gn].float().reshape(m, groups, n_state).repeat_interleave(heads // groups, dim=1)
+    C = xbc[:, inner + gn:].float().reshape(m, groups, n_state).repeat_interleave(heads // groups, dim=1)
+    d = torch.nn.functional.softplus(dt.float() + dt_bias, threshold=1e9)
+    decay = torch.exp(-torch.exp(a_log)[None, :] * d)
+    y = torch.empty((m, heads, head_dim), dtype=torch.float32, device=xbc.device)
+    for i in range(len(cu_rows) - 1):
+        slot = int(slot_ids[i])
+        S = state[slot].clone()
+        for r in range(int(cu_rows[i]), int(cu_rows[i + 1])):
+            S = decay[r][:, None, None] * S + (d[r][:, None] * B[r])[:, :, None] * x[r][:, None, :]
+            y[r] = torch.einsum("hnp,hn->hp", S, C[r]) + skip[:, None] * x[r]
+        state[slot] = S
+    zf = z.float()
+    return y.reshape(m, inner) * (zf * torch.sigmoid(zf))
+
+
+def pair_norm_mean(a, b, gain_a, gain_b, eps):
+    return 0.5 * (_norm(a, gain_a, eps) + _norm(b, gain_b, eps))
+
+
+def mul_sigmoid(x, g):
+    x.copy_((x.float() * torch.sigmoid(g.float())).to(x.dtype))
+    return x
 
 
 def gather_rows(x, rows):

@@ -87,7 +87,9 @@ __device__ __forceinline__ float gelu_tanh_fast(float g) {
 // The activations offered are of one form, act(g) = g / (1 + 2^(g (c1 + c3 g^2))): gelu-tanh (above) with
 // c1 = -2 * 0.7978845608 * log2(e), c3 = c1 * 0.044715, and SiLU, g / (1 + e^-g), with c1 = -log2(e), c3 = 0.  The
 // bf16 products' epilogues take the two constants (`epi.x`, `epi.y`) and have no branch on the activation's kind.
-enum { TP_ACT_GELU_TANH = 0, TP_ACT_SILU = 1 };
+// ReLU is the limit of the form for c1 -> -infinity: with c1 = -1e30 the power of two is 0 for every g above 1e-28
+// and infinite for every g below -1e-28, so the quotient is g or -0 (and within 1e-28 of 0 in between).
+enum { TP_ACT_GELU_TANH = 0, TP_ACT_SILU = 1, TP_ACT_RELU = 2 };
 // which elements of a head a rotation pairs: (f, f + rotary_dim / 2) as the reference does
 // (runtime/cuda/codebook_gemv.cu:219-230), or neighbours (2f, 2f + 1)
 enum { TP_ROPE_HALVES = 0, TP_ROPE_NEIGHBOURS = 1 };
@@ -95,6 +97,7 @@ static inline bool tp_gate_constants(int act, float* c1, float* c3) {
     constexpr float LOG2E = 1.4426950408889634f;
     if (act == TP_ACT_GELU_TANH) { *c1 = -2.f * 0.7978845608f * LOG2E; *c3 = *c1 * 0.044715f; return true; }
     if (act == TP_ACT_SILU) { *c1 = -LOG2E; *c3 = 0.f; return true; }
+    if (act == TP_ACT_RELU) { *c1 = -1e30f; *c3 = 0.f; return true; }
     return false;
 }
 __device__ __forceinline__ float gate_act_fast(float g, float2 epi) {
@@ -102,5 +105,5 @@ __device__ __forceinline__ float gate_act_fast(float g, float2 epi) {
 }
 // the same in full float32 arithmetic, for the float32 path
 __device__ __forceinline__ float gate_act_exact(float g, int act) {
-    return act == TP_ACT_SILU ? g / (1.f + expf(-g)) : gelu_tanh_f(g);
+    return act == TP_ACT_SILU ? g / (1.f + expf(-g)) : (act == TP_ACT_RELU ? fmaxf(g, 0.f) : gelu_tanh_f(g));
 }

@@ -673,7 +673,7 @@ __global__ void gated_act_k(const float* __restrict__ y, T* __restrict__ out, in
 
 extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, int act, void* stream) {
     TP_REQUIRE(M > 0 && I > 0, "gated_act: empty shape M=%d I=%d", M, I);
-    TP_REQUIRE(act == TP_ACT_GELU_TANH || act == TP_ACT_SILU, "gated_act: unknown activation %d", act);
+    TP_REQUIRE(act == TP_ACT_GELU_TANH || act == TP_ACT_SILU || act == TP_ACT_RELU, "gated_act: unknown activation %d", act);
     const int Ip2 = 2 * ((I + 15) / 16) * 16;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TP_BF16) gated_act_k<bf16_t><<<M, 256, 0, s>>>(y, (bf16_t*)out, I, Ip2, act);

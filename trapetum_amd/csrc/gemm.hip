@@ -101,7 +101,7 @@ static int check_args(const GemmArgs& a) {
         const int padded = 2 * ((a.units + 15) / 16) * 16;
         TP_REQUIRE(a.units > 0 && a.N == padded, "gated product: %d units need a packed matrix of %d rows, found %d", a.units, padded, a.N);
         float c1, c3;
-        TP_REQUIRE(tp_gate_constants(a.act, &c1, &c3), "gated product: activation %d is neither gelu-tanh (%d) nor SiLU (%d)", a.act, TP_ACT_GELU_TANH, TP_ACT_SILU);
+        TP_REQUIRE(tp_gate_constants(a.act, &c1, &c3), "gated product: activation %d is none of gelu-tanh (%d), SiLU (%d), ReLU (%d)", a.act, TP_ACT_GELU_TANH, TP_ACT_SILU, TP_ACT_RELU);
     }
     return 0;
 }

@@ -5,19 +5,25 @@
 #include "tile.h"
 #include "tile_mfma.h"
 
-// ---- scores = softmax(logits) over all experts; the `top` largest (ties: the smaller index) and their scores --------
-// grid (rows), one wave a row; dynamic LDS: E floats
+// ---- scores = softmax(logits) over all experts, or sigmoid(logits) of each; the `top` largest (ties: the smaller
+// index) and their scores.  grid (rows), one wave a row; dynamic LDS: E floats
+enum { TP_ROUTE_SOFTMAX = 0, TP_ROUTE_SIGMOID = 1 };
 __global__ void __launch_bounds__(64)
-route_top_k(const float* __restrict__ logits, int E, int top, int renormalize, int* __restrict__ chosen, float* __restrict__ weight) {
+route_top_k(const float* __restrict__ logits, int E, int top, int renormalize, int score, int* __restrict__ chosen, float* __restrict__ weight) {
     extern __shared__ float sc[];
     const int r = blockIdx.x, lane = threadIdx.x;
     const float* z = logits + (size_t)r * E;
-    float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
-    mx = wave_max(mx);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += 64) { const float p = expf(z[e] - mx); sc[e] = p; sum += p; }
-    sum = wave_sum(sum);
+    float sum = 1.f;
+    if (score == TP_ROUTE_SIGMOID) {
+        for (int e = lane; e < E; e += 64) sc[e] = 1.f / (1.f + expf(-z[e]));
+    } else {
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+        mx = wave_max(mx);
+        sum = 0.f;
+        for (int e = lane; e < E; e += 64) { const float p = expf(z[e] - mx); sc[e] = p; sum += p; }
+        sum = wave_sum(sum);
+    }
     __syncthreads();
     float kept = 0.f;
     for (int k = 0; k < top; k++) {
@@ -42,11 +48,12 @@ route_top_k(const float* __restrict__ logits, int E, int top, int renormalize, i
         for (int k = 0; k < top; k++) weight[(size_t)r * top + k] /= kept;
 }
 
-extern "C" int tp_route_top(const float* logits, int M, int E, int top, int renormalize, int* chosen, float* weight, void* stream) {
+extern "C" int tp_route_top(const float* logits, int M, int E, int top, int renormalize, int score, int* chosen, float* weight, void* stream) {
+    TP_REQUIRE(score == TP_ROUTE_SOFTMAX || score == TP_ROUTE_SIGMOID, "route_top: unknown kind of score %d", score);
     TP_REQUIRE(M > 0 && E > 0 && top > 0 && top <= E, "route_top: %d of %d experts for %d rows", top, E, M);
     TP_REQUIRE(logits && chosen && weight, "route_top: a null operand");
     TP_REQUIRE((size_t)E * sizeof(float) <= 60000, "route_top: %d experts exceed the kernel's table", E);
-    route_top_k<<<M, 64, (size_t)E * sizeof(float), (hipStream_t)stream>>>(logits, E, top, renormalize, chosen, weight);
+    route_top_k<<<M, 64, (size_t)E * sizeof(float), (hipStream_t)stream>>>(logits, E, top, renormalize, score, chosen, weight);
     return tp_check_launch("route_top");
 }
 
@@ -91,7 +98,7 @@ expert_sort_k(const int* __restrict__ chosen, int P, int E, int* __restrict__ or
 template <typename T, bool GATED, int TM>
 __global__ void __launch_bounds__(256)
 expert_linear_k(const T* __restrict__ a, const T* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
-                int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out) {
+                int E, int top, int N, int K, float limit, float alpha, float shift, const float* __restrict__ in_scale, void* __restrict__ out) {
     constexpr int TN = 64, BK = 16;
     __shared__ TileShared<TM, GATED ? 2 * TN : TN, BK> sh;
     int t = blockIdx.y, e = 0, lo = 0, hi = 0;
@@ -116,7 +123,8 @@ expert_linear_k(const T* __restrict__ a, const T* __restrict__ w, const int* __r
             for (int j = 0; j < TN / 16; j++) {
                 const int p = p0 + ty + 16 * i, n = n0 + tx + 16 * j;
                 if (p >= hi || n >= N) continue;
-                const float g = fminf(acc[i][j], limit), u = fminf(fmaxf(acc[i][j + TN / 16], -limit), limit);
+                const float sc = in_scale ? in_scale[order[p]] : 1.f;      // the pair's weight on the expert's input: W (s h) = s (W h)
+                const float g = fminf(acc[i][j] * sc, limit), u = fminf(fmaxf(acc[i][j + TN / 16] * sc, -limit), limit);
                 st_f32((T*)out + (size_t)p * N + n, g / (1.f + expf(-alpha * g)) * (u + shift));
             }
     } else {
@@ -139,7 +147,7 @@ expert_linear_k(const T* __restrict__ a, const T* __restrict__ w, const int* __r
 template <int MODE, int TM>
 __global__ void __launch_bounds__(256)
 expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
-                     int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out, int k_slice, long out_slice) {
+                     int E, int top, int N, int K, float limit, float alpha, float shift, const float* __restrict__ in_scale, void* __restrict__ out, int k_slice, long out_slice) {
     constexpr bool GATED = MODE == 1;
     constexpr int COLS = MODE == 2 ? 128 : 64;
     using Tile = MfmaTile<TM, MODE != 0>;
@@ -180,10 +188,11 @@ expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
             if (p >= hi) continue;
             if constexpr (GATED) {
                 const int n = n0 + Tile::n_of(j);
+                const float sc = in_scale ? in_scale[order[p]] : 1.f;
                 bf16_t o[4];
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const float g = fminf(tile.acc[0][i][j][v], limit), u = fminf(fmaxf(tile.acc[1][i][j][v], -limit), limit);
+                    const float g = fminf(tile.acc[0][i][j][v] * sc, limit), u = fminf(fmaxf(tile.acc[1][i][j][v] * sc, -limit), limit);
                     o[v] = f32_to_bf16(g / (1.f + expf(-alpha * g)) * (u + shift));
                 }
                 bf16_t* dst = (bf16_t*)out + (size_t)p * N + n;
@@ -222,7 +231,7 @@ expert_linear_mfma_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
 template <bool GATED>
 __global__ void __launch_bounds__(256, 2)
 expert_direct_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
-                int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out) {
+                int E, int top, int N, int K, float limit, float alpha, float shift, const float* __restrict__ in_scale, void* __restrict__ out) {
     constexpr int BM = 128, BN = 128, BK = 64, LDS = BK, TM = 4, TN = 4;
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
@@ -311,13 +320,14 @@ expert_direct_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, cons
         const int p = p0 + wm * 64 + i * 16 + r;
         if (p >= hi) continue;
         if constexpr (GATED) {
+            const float sc = in_scale ? in_scale[order[p]] : 1.f;
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const int n = n0 + wn * 32 + j * 16 + g * 4;
                 bf16_t o[4];
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const float gg = fminf(acc[i][j][v], limit), uu = fminf(fmaxf(acc[i][j + 2][v], -limit), limit);
+                    const float gg = fminf(acc[i][j][v] * sc, limit), uu = fminf(fmaxf(acc[i][j + 2][v] * sc, -limit), limit);
                     o[v] = f32_to_bf16(gg / (1.f + expf(-alpha * gg)) * (uu + shift));
                 }
                 bf16_t* dst = (bf16_t*)out + (size_t)p * N + n;
@@ -353,7 +363,7 @@ expert_direct_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, cons
 template <bool GATED>
 __global__ void __launch_bounds__(256)
 expert_stream_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ order, const int* __restrict__ first,
-                int E, int top, int N, int K, float limit, float alpha, float shift, void* __restrict__ out, int k_slice, long out_slice) {
+                int E, int top, int N, int K, float limit, float alpha, float shift, const float* __restrict__ in_scale, void* __restrict__ out, int k_slice, long out_slice) {
     constexpr int TM = 16, UN = 8;
     int t = blockIdx.y, e = 0, lo = 0, hi = 0;
     for (; e < E; e++) {
@@ -398,10 +408,11 @@ expert_stream_k(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, cons
     const int n = n0 + g * 4;
     if constexpr (GATED) {
         bf16_t* dst = (bf16_t*)out + (size_t)p * N + n;
+        const float sc = in_scale ? in_scale[order[p]] : 1.f;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             if (n + v >= N) continue;
-            const float gg = fminf(acc_g[v], limit), uu = fminf(fmaxf(acc_u[v], -limit), limit);
+            const float gg = fminf(acc_g[v] * sc, limit), uu = fminf(fmaxf(acc_u[v] * sc, -limit), limit);
             dst[v] = f32_to_bf16(gg / (1.f + expf(-alpha * gg)) * (uu + shift));
         }
     } else {
@@ -424,7 +435,7 @@ expert_combine_k(const float* __restrict__ pair_out, int n_slices, long slice_st
         const float* src = pair_out + (size_t)place[(size_t)m * top + k] * D + d;
         float v = src[0];
         for (int z = 1; z < n_slices; z++) v += src[(size_t)z * slice_stride];       // the K slices of a pair's output, in slice order
-        acc = __builtin_fmaf(weight[(size_t)m * top + k], v, acc);
+        acc = weight ? __builtin_fmaf(weight[(size_t)m * top + k], v, acc) : acc + v;
     }
     out[(size_t)m * D + d] = acc;
 }
@@ -437,8 +448,11 @@ extern "C" long tp_expert_ffn_workspace_bytes(int dtype, int M, int top, int E, 
 }
 
 extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* chosen, const float* weight, int top, int E, int F,
-                             const void* w_gate_up, const void* w_down, float limit, float alpha, float shift,
+                             const void* w_gate_up, const void* w_down, float limit, float alpha, float shift, int weight_input,
                              void* workspace, long workspace_bytes, float* out, int plain, void* stream) {
+    // weight_input: a pair's weight multiplies the expert's input (inside the activation) instead of its output
+    const float* in_scale = weight_input ? weight : nullptr;
+    const float* out_weight = weight_input ? nullptr : weight;
     TP_REQUIRE(M > 0 && D > 0 && top > 0 && E > 0 && F > 0, "expert_ffn: empty shape M=%d D=%d top=%d E=%d F=%d", M, D, top, E, F);
     TP_REQUIRE(x && chosen && weight && w_gate_up && w_down && workspace && out, "expert_ffn: a null operand");
     TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F32, "expert_ffn: unknown dtype %d", dtype);
@@ -461,37 +475,37 @@ extern "C" int tp_expert_ffn(const void* x, int dtype, int M, int D, const int* 
     const int TM = few ? 16 : (many ? 128 : 64);
     const int row_tiles = tp_cdiv(P, TM) + (E < P ? E : P);
     TP_REQUIRE(row_tiles <= 65535, "expert_ffn: %d row tiles exceed one launch", row_tiles);
-#define TP_EXPERT(T, G, TMv, Nv, Kv, A, W, O) expert_linear_k<T, G, TMv><<<dim3(tp_cdiv(Nv, 64), row_tiles), 256, 0, s>>>( \
-        (const T*)(A), (const T*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O)
-#define TP_EXPERT_MFMA(G, TMv, Nv, Kv, A, W, O, Z) expert_linear_mfma_k<G, TMv><<<dim3(tp_cdiv(Nv, (G) == 2 ? 128 : 64), row_tiles, Z), 256, 0, s>>>( \
-        (const bf16_t*)(A), (const bf16_t*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, O, (Kv) / (Z), (long)P * (Nv))
+#define TP_EXPERT(T, G, TMv, Nv, Kv, A, W, S, O) expert_linear_k<T, G, TMv><<<dim3(tp_cdiv(Nv, 64), row_tiles), 256, 0, s>>>( \
+        (const T*)(A), (const T*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, S, O)
+#define TP_EXPERT_MFMA(G, TMv, Nv, Kv, A, W, S, O, Z) expert_linear_mfma_k<G, TMv><<<dim3(tp_cdiv(Nv, (G) == 2 ? 128 : 64), row_tiles, Z), 256, 0, s>>>( \
+        (const bf16_t*)(A), (const bf16_t*)(W), order, first, E, top, Nv, Kv, limit, alpha, shift, S, O, (Kv) / (Z), (long)P * (Nv))
     if (cores) {
         if (few) expert_stream_k<true><<<dim3(tp_cdiv(F, 64), row_tiles, 1), 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w_gate_up, order, first, E, top, F, D,
-                                                                                             limit, alpha, shift, y, D, 0);
+                                                                                             limit, alpha, shift, in_scale, y, D, 0);
         else if (many && D % 64 == 0 && (long)M * D * 2 < (1L << 32) && 2L * F * D * 2 < (1L << 32))
             expert_direct_k<true><<<dim3(tp_cdiv(F, 64), row_tiles), 256, 0, s>>>((const bf16_t*)x, (const bf16_t*)w_gate_up, order, first, E, top, F, D,
-                                                                                  limit, alpha, shift, y);
-        else if (many) TP_EXPERT_MFMA(1, 128, F, D, x, w_gate_up, y, 1); else TP_EXPERT_MFMA(1, 64, F, D, x, w_gate_up, y, 1);
+                                                                                  limit, alpha, shift, in_scale, y);
+        else if (many) TP_EXPERT_MFMA(1, 128, F, D, x, w_gate_up, in_scale, y, 1); else TP_EXPERT_MFMA(1, 64, F, D, x, w_gate_up, in_scale, y, 1);
         if (int rc = tp_check_launch("expert_ffn (gate, up; matrix cores)")) return rc;
         const int zs = down_slices(P, F);
         if (few) expert_stream_k<false><<<dim3(tp_cdiv(D, 64), row_tiles, zs), 256, 0, s>>>((const bf16_t*)y, (const bf16_t*)w_down, order, first, E, top, D, F,
-                                                                                               limit, alpha, shift, pair_out, F / zs, (long)P * D);
+                                                                                               limit, alpha, shift, nullptr, pair_out, F / zs, (long)P * D);
         else if (many && F % 64 == 0 && (long)P * F * 2 < (1L << 32) && (long)D * F * 2 < (1L << 32))
             expert_direct_k<false><<<dim3(tp_cdiv(D, 128), row_tiles), 256, 0, s>>>((const bf16_t*)y, (const bf16_t*)w_down, order, first, E, top, D, F,
-                                                                                    limit, alpha, shift, pair_out);
-        else if (many) TP_EXPERT_MFMA(2, 128, D, F, y, w_down, pair_out, 1); else TP_EXPERT_MFMA(0, 64, D, F, y, w_down, pair_out, 1);
+                                                                                    limit, alpha, shift, nullptr, pair_out);
+        else if (many) TP_EXPERT_MFMA(2, 128, D, F, y, w_down, nullptr, pair_out, 1); else TP_EXPERT_MFMA(0, 64, D, F, y, w_down, nullptr, pair_out, 1);
         if (int rc = tp_check_launch("expert_ffn (down; matrix cores)")) return rc;
-        expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, zs, (long)P * D, place, weight, top, D, out);
+        expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, zs, (long)P * D, place, out_weight, top, D, out);
         return tp_check_launch("expert_ffn (combine)");
     }
 #undef TP_EXPERT_MFMA
-    if (dtype == TP_BF16) { if (few) TP_EXPERT(bf16_t, true, 16, F, D, x, w_gate_up, y); else TP_EXPERT(bf16_t, true, 64, F, D, x, w_gate_up, y); }
-    else { if (few) TP_EXPERT(float, true, 16, F, D, x, w_gate_up, y); else TP_EXPERT(float, true, 64, F, D, x, w_gate_up, y); }
+    if (dtype == TP_BF16) { if (few) TP_EXPERT(bf16_t, true, 16, F, D, x, w_gate_up, in_scale, y); else TP_EXPERT(bf16_t, true, 64, F, D, x, w_gate_up, in_scale, y); }
+    else { if (few) TP_EXPERT(float, true, 16, F, D, x, w_gate_up, in_scale, y); else TP_EXPERT(float, true, 64, F, D, x, w_gate_up, in_scale, y); }
     if (int rc = tp_check_launch("expert_ffn (gate, up)")) return rc;
-    if (dtype == TP_BF16) { if (few) TP_EXPERT(bf16_t, false, 16, D, F, y, w_down, pair_out); else TP_EXPERT(bf16_t, false, 64, D, F, y, w_down, pair_out); }
-    else { if (few) TP_EXPERT(float, false, 16, D, F, y, w_down, pair_out); else TP_EXPERT(float, false, 64, D, F, y, w_down, pair_out); }
+    if (dtype == TP_BF16) { if (few) TP_EXPERT(bf16_t, false, 16, D, F, y, w_down, nullptr, pair_out); else TP_EXPERT(bf16_t, false, 64, D, F, y, w_down, nullptr, pair_out); }
+    else { if (few) TP_EXPERT(float, false, 16, D, F, y, w_down, nullptr, pair_out); else TP_EXPERT(float, false, 64, D, F, y, w_down, nullptr, pair_out); }
 #undef TP_EXPERT
     if (int rc = tp_check_launch("expert_ffn (down)")) return rc;
-    expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, 1, 0, place, weight, top, D, out);
+    expert_combine_k<<<dim3(M, tp_cdiv(D, 256)), 256, 0, s>>>(pair_out, 1, 0, place, out_weight, top, D, out);
     return tp_check_launch("expert_ffn (combine)");
 }

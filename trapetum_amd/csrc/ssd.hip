@@ -1,0 +1,305 @@
+// A state-space mixer's own kernels (a decaying matrix state per head, after a short convolution), and the two small
+// row-wise kernels of a mixer that runs two mixers side by side.
+//
+//   conv_act      out_t = act(b + sum_j w[:, j] u_(t - taps + 1 + j)) on every channel of the step's rows, the rows before
+//                 the step kept per sequence as a state (float32, the projection's values as they were)
+//   ssd_scan      S_t = exp(-exp(a) dt_t) S_(t-1) + dt_t B_t x_t^T,  y_t = (S_t^T C_t + D x_t) * silu(z_t),
+//                 dt_t = softplus(raw_t + bias); S, dt, the decay and y in float32
+//   pair_norm_mean  0.5 (a / rms(a) * wa + b / rms(b) * wb) over rows
+//   mul_sigmoid   x *= sigmoid(g)
+#include "common.h"
+
+enum { TP_CONV_ACT_NONE = 0, TP_CONV_ACT_SILU = 1 };
+
+// grid (rows, channel blocks of 256).  wt: taps transposed [taps, C].  state [slots, taps - 1, C], oldest row first.
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256)
+conv_act_k(const TI* __restrict__ x, long x_stride, const float* __restrict__ wt, const float* __restrict__ bias,
+           float* __restrict__ state, const int* __restrict__ slot_ids, const int* __restrict__ cu_rows,
+           const int* __restrict__ row_seq, TO* __restrict__ out, long out_stride, int C, int taps, int act, int one_row_each) {
+    const int r = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int seq = row_seq[r], i = r - cu_rows[seq], S = taps - 1;
+    float* st = S > 0 ? state + (size_t)slot_ids[seq] * S * C + c : nullptr;
+    const float xr = ld_f32(x + (size_t)r * x_stride + c);
+    float acc = bias ? bias[c] : 0.f;
+    for (int j = 0; j < taps; j++) {
+        const int src = i - (S - j);                     // the step's row this tap reads; negative: before the step
+        const float v = j == S ? xr : (src >= 0 ? ld_f32(x + (size_t)(r - (S - j)) * x_stride + c) : st[(size_t)(S + src) * C]);
+        acc = __builtin_fmaf(wt[(size_t)j * C + c], v, acc);
+    }
+    if (act == TP_CONV_ACT_SILU) acc = acc / (1.f + expf(-acc));
+    st_f32(out + (size_t)r * out_stride + c, acc);
+    if (one_row_each && S > 0) {
+        for (int s = 0; s + 1 < S; s++) st[(size_t)s * C] = st[(size_t)(s + 1) * C];
+        st[(size_t)(S - 1) * C] = xr;
+    }
+}
+
+// grid (sequences, channel blocks): the state takes the last taps - 1 rows of (state, the step's rows)
+template <typename TI>
+__global__ void __launch_bounds__(256)
+conv_act_state_k(const TI* __restrict__ x, long x_stride, float* __restrict__ state, const int* __restrict__ slot_ids,
+                 const int* __restrict__ cu_rows, int C, int taps) {
+    const int seq = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int first = cu_rows[seq], count = cu_rows[seq + 1] - first, S = taps - 1;
+    float* st = state + (size_t)slot_ids[seq] * S * C + c;
+    for (int s = 0; s < S; s++) {                        // ascending: a row of the old state is read before it is overwritten
+        const int src = count - S + s;
+        st[(size_t)s * C] = src >= 0 ? ld_f32(x + (size_t)(first + src) * x_stride + c) : st[(size_t)(s + count) * C];
+    }
+}
+
+extern "C" int tp_conv_act(const void* x, long x_stride, int in_dtype, const float* wt, const float* bias, float* state,
+                           const int* slot_ids, const int* cu_rows, const int* row_seq, void* out, long out_stride, int out_dtype,
+                           int M, int n_seq, int C, int taps, int act, int one_row_each, void* stream) {
+    TP_REQUIRE(M > 0 && n_seq > 0 && C > 0 && taps >= 1, "conv_act: empty shape M=%d sequences=%d C=%d taps=%d", M, n_seq, C, taps);
+    TP_REQUIRE(x && wt && out && cu_rows && row_seq, "conv_act: a null operand");
+    TP_REQUIRE(taps == 1 || (state && slot_ids), "conv_act: %d taps need the sequences' states", taps);
+    TP_REQUIRE(!one_row_each || M == n_seq, "conv_act: one row each, but %d rows for %d sequences", M, n_seq);
+    TP_REQUIRE(act == TP_CONV_ACT_NONE || act == TP_CONV_ACT_SILU, "conv_act: unknown activation %d", act);
+    TP_REQUIRE(in_dtype == out_dtype && (in_dtype == TP_BF16 || in_dtype == TP_F32), "conv_act: rows and output share one dtype, bfloat16 or float32");
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(M, tp_cdiv(C, 256));
+    if (in_dtype == TP_BF16)
+        conv_act_k<bf16_t, bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, x_stride, wt, bias, state, slot_ids, cu_rows, row_seq, (bf16_t*)out, out_stride, C, taps, act, one_row_each);
+    else
+        conv_act_k<float, float><<<grid, 256, 0, s>>>((const float*)x, x_stride, wt, bias, state, slot_ids, cu_rows, row_seq, (float*)out, out_stride, C, taps, act, one_row_each);
+    if (int rc = tp_check_launch("conv_act")) return rc;
+    if (taps > 1 && !one_row_each) {
+        dim3 sgrid(n_seq, tp_cdiv(C, 256));
+        if (in_dtype == TP_BF16) conv_act_state_k<bf16_t><<<sgrid, 256, 0, s>>>((const bf16_t*)x, x_stride, state, slot_ids, cu_rows, C, taps);
+        else conv_act_state_k<float><<<sgrid, 256, 0, s>>>((const float*)x, x_stride, state, slot_ids, cu_rows, C, taps);
+        return tp_check_launch("conv_act (state)");
+    }
+    return 0;
+}
+
+// ---- the scan ---------------------------------------------------------------------------------------------------
+struct SsdArgs {
+    const void* xbc; long xbc_stride;                    // rows [x: heads P | B: groups N | C: groups N] after convolution and activation
+    const void* z; long z_stride;                        // gate rows [heads P]
+    const void* dt; long dt_stride;                      // raw step sizes [heads]
+    const float* dt_bias; const float* a_log; const float* skip;
+    float* state;                                        // [slots, heads, N, P]
+    const int* slot_ids; const int* cu_rows;
+    float* y;                                            // [rows, heads P]
+    int heads, groups, N, P;
+    // a scan cut into pieces (chunk > 0): piece c of a sequence covers its rows [c chunk, (c + 1) chunk)
+    int chunk, max_chunks;
+    float* carry;                                        // [sequences, max_chunks, heads, N, P]: the state a piece ends with, started from zero
+    float* decay;                                        // [sequences, max_chunks, heads]: the product of its rows' decays
+};
+
+__device__ __forceinline__ float softplus_f(float v) { return log1pf(expf(-fabsf(v))) + fmaxf(v, 0.f); }
+
+// One wave owns 64 value channels of one head of one sequence (or of one piece of it): lane p keeps column p of the
+// state, NR elements, in registers; the rows' B and C vectors, step sizes, decays, inputs and gates are staged in LDS
+// TC rows at a time (every load of a round is asked for at once), and a row then costs the lane 2 N multiply-adds
+// with no traffic between lanes.  FULL: N == NR, no bounds in the inner loop.
+// MODE 0: the whole scan from the slot's state, which it leaves updated.
+// MODE 1: a piece (not the last) from a zero state: writes the state it ends with and its total decay, no outputs.
+// MODE 2: a piece from the state `carry` holds for its start: writes outputs; the last piece leaves the slot's state.
+template <typename T, int NR, int MODE, bool FULL>
+__global__ void __launch_bounds__(64)
+ssd_scan_k(SsdArgs a) {
+    constexpr int TC = 16;
+    extern __shared__ float lds[];                       // B [TC][N], C [TC][N], dt [TC], decay [TC], x [TC][64], z [TC][64]
+    const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int pieces_z = MODE == 0 ? 1 : a.max_chunks;
+    const int piece = MODE == 0 ? 0 : blockIdx.z % pieces_z, pc = MODE == 0 ? blockIdx.z : blockIdx.z / pieces_z;
+    const int p = pc * 64 + lane;
+    const bool live = p < a.P;
+    const int N = FULL ? NR : a.N, P = a.P, g = head / (a.heads / a.groups);
+    const int first = a.cu_rows[seq], count = a.cu_rows[seq + 1] - first;
+    int r0 = first, r1 = first + count;
+    if (MODE != 0) {
+        r0 = first + piece * a.chunk;
+        r1 = min(r0 + a.chunk, first + count);
+        if (r0 >= r1) return;
+    }
+    const bool last_piece = MODE == 0 || r1 == first + count;
+    if (MODE == 1 && last_piece) return;                 // nobody starts from the state the last piece ends with
+    float* Bs = lds; float* Cs = lds + TC * N; float* dts = Cs + TC * N; float* dec = dts + TC;
+    float* xs = dec + TC; float* zs = xs + TC * 64;
+    const float rate = expf(a.a_log[head]), bias = a.dt_bias[head], skip = a.skip[head];
+    float S[NR];
+    float* slot_state = a.state + (((size_t)a.slot_ids[seq] * a.heads + head) * N) * P + p;
+    const float* from = slot_state;
+    if (MODE == 2) from = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
+#pragma unroll
+    for (int n = 0; n < NR; n++) S[n] = (MODE != 1 && live && (FULL || n < N)) ? from[(size_t)n * P] : 0.f;
+    float total = 1.f;
+    const size_t inner = (size_t)a.heads * P;
+    for (int t0 = r0; t0 < r1; t0 += TC) {
+        const int tn = min(TC, r1 - t0);
+        __syncthreads();
+        for (int i = lane; i < tn * N; i += 64) {
+            const int t = i / N, n = i - t * N;
+            const T* row = (const T*)a.xbc + (size_t)(t0 + t) * a.xbc_stride + inner + (size_t)g * N + n;
+            Bs[i] = ld_f32(row);
+            Cs[i] = ld_f32(row + (size_t)a.groups * N);
+        }
+        for (int t = 0; t < tn; t++) {
+            const size_t r = (size_t)(t0 + t);
+            xs[t * 64 + lane] = live ? ld_f32((const T*)a.xbc + r * a.xbc_stride + (size_t)head * P + p) : 0.f;
+            if (MODE != 1) zs[t * 64 + lane] = live ? ld_f32((const T*)a.z + r * a.z_stride + (size_t)head * P + p) : 0.f;
+        }
+        if (lane < tn) {
+            const float d = softplus_f(ld_f32((const T*)a.dt + (size_t)(t0 + lane) * a.dt_stride + head) + bias);
+            dts[lane] = d;
+            dec[lane] = expf(-rate * d);
+        }
+        __syncthreads();
+        for (int t = 0; t < tn; t++) {
+            const float x = xs[t * 64 + lane];
+            const float d = dec[t], dx = dts[t] * x;
+            const float* Bt = Bs + t * N; const float* Ct = Cs + t * N;
+            float acc = 0.f;
+#pragma unroll
+            for (int n = 0; n < NR; n++) {
+                if (FULL || n < N) {
+                    S[n] = __builtin_fmaf(d, S[n], dx * Bt[n]);
+                    if (MODE != 1) acc = __builtin_fmaf(S[n], Ct[n], acc);
+                }
+            }
+            if (MODE == 1) total *= d;
+            else if (live) {
+                const float zz = zs[t * 64 + lane];
+                a.y[(size_t)(t0 + t) * inner + (size_t)head * P + p] = __builtin_fmaf(skip, x, acc) * (zz / (1.f + expf(-zz)));
+            }
+        }
+    }
+    if (MODE == 1) {
+        float* to = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
+        if (live) {
+#pragma unroll
+            for (int n = 0; n < NR; n++) if (FULL || n < N) to[(size_t)n * P] = S[n];
+        }
+        if (pc == 0 && lane == 0) a.decay[((size_t)seq * a.max_chunks + piece) * a.heads + head] = total;
+    } else if (last_piece && live) {
+#pragma unroll
+        for (int n = 0; n < NR; n++) if (FULL || n < N) slot_state[(size_t)n * P] = S[n];
+    }
+}
+
+// The states at the pieces' starts from the pieces' own end states: walking the pieces, carry[c] (what piece c ends
+// with when started from zero) gives way to the state piece c starts from, s, and s <- decay[c] s + carry[c].
+// grid (sequences, heads, blocks of N P / 256)
+__global__ void __launch_bounds__(256)
+ssd_carry_k(SsdArgs a) {
+    const int seq = blockIdx.x, head = blockIdx.y;
+    const int e = blockIdx.z * 256 + threadIdx.x, NP = a.N * a.P;
+    if (e >= NP) return;
+    const int count = a.cu_rows[seq + 1] - a.cu_rows[seq];
+    const int pieces = (count + a.chunk - 1) / a.chunk;
+    float s = a.state[((size_t)a.slot_ids[seq] * a.heads + head) * NP + e];
+    for (int c = 0; c < pieces; c++) {
+        float* at = a.carry + (((size_t)seq * a.max_chunks + c) * a.heads + head) * NP + e;
+        const float ended = c + 1 < pieces ? *at : 0.f;  // the last piece wrote none
+        *at = s;
+        if (c + 1 < pieces) s = __builtin_fmaf(a.decay[((size_t)seq * a.max_chunks + c) * a.heads + head], s, ended);
+    }
+}
+
+template <typename T, int MODE>
+static int launch_scan(const SsdArgs& a, dim3 grid, size_t lds, hipStream_t s) {
+#define TP_SSD(NR) do { if (a.N == NR) ssd_scan_k<T, NR, MODE, true><<<grid, 64, lds, s>>>(a); else ssd_scan_k<T, NR, MODE, false><<<grid, 64, lds, s>>>(a); } while (0)
+    if (a.N <= 16) TP_SSD(16);
+    else if (a.N <= 32) TP_SSD(32);
+    else if (a.N <= 64) TP_SSD(64);
+    else if (a.N <= 128) TP_SSD(128);
+    else TP_SSD(256);
+#undef TP_SSD
+    return tp_check_launch("ssd_scan");
+}
+
+extern "C" long tp_ssd_scan_workspace_bytes(int n_seq, int max_count, int heads, int N, int P, int chunk) {
+    if (chunk <= 0 || max_count <= chunk) return 0;
+    const long pieces = (max_count + chunk - 1) / chunk;
+    return (long)n_seq * pieces * heads * ((long)N * P + 1) * (long)sizeof(float);
+}
+
+// chunk 0: one pass per sequence.  chunk > 0 and a sequence longer than it: three passes over pieces of `chunk` rows.
+extern "C" int tp_ssd_scan(const void* xbc, long xbc_stride, const void* z, long z_stride, const void* dt, long dt_stride, int dtype,
+                           const float* dt_bias, const float* a_log, const float* skip, float* state, const int* slot_ids,
+                           const int* cu_rows, float* y, int n_seq, int max_count, int heads, int groups, int N, int P,
+                           int chunk, void* workspace, long workspace_bytes, void* stream) {
+    TP_REQUIRE(n_seq > 0 && max_count > 0 && heads > 0 && groups > 0 && N > 0 && P > 0, "ssd_scan: empty shape sequences=%d heads=%d groups=%d N=%d P=%d", n_seq, heads, groups, N, P);
+    TP_REQUIRE(heads % groups == 0, "ssd_scan: %d heads are no multiple of %d groups", heads, groups);
+    TP_REQUIRE(N <= 256, "ssd_scan: a state of %d rows per head exceeds 256", N);
+    TP_REQUIRE(heads <= 65535 && (P + 63) / 64 <= 65535, "ssd_scan: too many heads or channels for one launch");
+    TP_REQUIRE(xbc && z && dt && dt_bias && a_log && skip && state && slot_ids && cu_rows && y, "ssd_scan: a null operand");
+    TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F32, "ssd_scan: unknown dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+    SsdArgs a{};
+    a.xbc = xbc; a.xbc_stride = xbc_stride; a.z = z; a.z_stride = z_stride; a.dt = dt; a.dt_stride = dt_stride;
+    a.dt_bias = dt_bias; a.a_log = a_log; a.skip = skip; a.state = state; a.slot_ids = slot_ids; a.cu_rows = cu_rows; a.y = y;
+    a.heads = heads; a.groups = groups; a.N = N; a.P = P;
+    const size_t lds = (size_t)(2 * 16 * N + 32 + 2 * 16 * 64) * sizeof(float);
+    const int pcs = (P + 63) / 64;
+    const long need = tp_ssd_scan_workspace_bytes(n_seq, max_count, heads, N, P, chunk);
+    if (need == 0) {
+        dim3 grid(n_seq, heads, pcs);
+        return dtype == TP_BF16 ? launch_scan<bf16_t, 0>(a, grid, lds, s) : launch_scan<float, 0>(a, grid, lds, s);
+    }
+    TP_REQUIRE(workspace && workspace_bytes >= need, "ssd_scan: a workspace of %ld bytes is too small (%ld)", workspace_bytes, need);
+    a.chunk = chunk; a.max_chunks = (max_count + chunk - 1) / chunk;
+    TP_REQUIRE((long)pcs * a.max_chunks <= 65535, "ssd_scan: %d pieces exceed one launch", a.max_chunks);
+    a.carry = (float*)workspace;
+    a.decay = a.carry + (size_t)n_seq * a.max_chunks * heads * N * P;
+    dim3 grid(n_seq, heads, pcs * a.max_chunks);
+    if (int rc = dtype == TP_BF16 ? launch_scan<bf16_t, 1>(a, grid, lds, s) : launch_scan<float, 1>(a, grid, lds, s)) return rc;
+    ssd_carry_k<<<dim3(n_seq, heads, tp_cdiv((long)N * P, 256)), 256, 0, s>>>(a);
+    if (int rc = tp_check_launch("ssd_scan (carry)")) return rc;
+    return dtype == TP_BF16 ? launch_scan<bf16_t, 2>(a, grid, lds, s) : launch_scan<float, 2>(a, grid, lds, s);
+}
+
+// ---- 0.5 (a / rms(a) * wa + b / rms(b) * wb), one block a row ------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+pair_norm_mean_k(const T* __restrict__ a, const T* __restrict__ b, const float* __restrict__ wa, const float* __restrict__ wb,
+                 float eps, float* __restrict__ out, int D) {
+    __shared__ float red[32];
+    const T* ar = a + (size_t)blockIdx.x * D; const T* br = b + (size_t)blockIdx.x * D;
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < D; i += 256) { const float x = ld_f32(ar + i), y = ld_f32(br + i); sa += x * x; sb += y * y; }
+    sa = block_sum_once(sa, red);
+    sb = block_sum_once(sb, red + 16);
+    const float ra = rsqrtf(sa / (float)D + eps), rb = rsqrtf(sb / (float)D + eps);
+    float* o = out + (size_t)blockIdx.x * D;
+    for (int i = threadIdx.x; i < D; i += 256) o[i] = 0.5f * ((ld_f32(ar + i) * ra) * wa[i] + (ld_f32(br + i) * rb) * wb[i]);
+}
+
+extern "C" int tp_pair_norm_mean(const void* a, const void* b, int dtype, const float* wa, const float* wb, float eps, float* out,
+                                 int M, int D, void* stream) {
+    TP_REQUIRE(M > 0 && D > 0 && a && b && wa && wb && out, "pair_norm_mean: empty shape or null operand (M=%d D=%d)", M, D);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TP_BF16) pair_norm_mean_k<bf16_t><<<M, 256, 0, s>>>((const bf16_t*)a, (const bf16_t*)b, wa, wb, eps, out, D);
+    else if (dtype == TP_F32) pair_norm_mean_k<float><<<M, 256, 0, s>>>((const float*)a, (const float*)b, wa, wb, eps, out, D);
+    else return tp_fail("pair_norm_mean: unknown dtype %d", dtype);
+    return tp_check_launch("pair_norm_mean");
+}
+
+// ---- x[r, c] *= sigmoid(g[r, c]) ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+mul_sigmoid_k(T* __restrict__ x, long x_stride, const T* __restrict__ g, long g_stride, int M, int C) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)M * C) return;
+    const long r = i / C, c = i - r * C;
+    T* xp = x + r * x_stride + c;
+    const float gv = ld_f32(g + r * g_stride + c);
+    st_f32(xp, ld_f32(xp) / (1.f + expf(-gv)));
+}
+
+extern "C" int tp_mul_sigmoid(void* x, long x_stride, const void* g, long g_stride, int dtype, int M, int C, void* stream) {
+    TP_REQUIRE(M > 0 && C > 0 && x && g, "mul_sigmoid: empty shape or null operand (M=%d C=%d)", M, C);
+    hipStream_t s = (hipStream_t)stream;
+    const int blocks = tp_cdiv((long)M * C, 256);
+    if (dtype == TP_BF16) mul_sigmoid_k<bf16_t><<<blocks, 256, 0, s>>>((bf16_t*)x, x_stride, (const bf16_t*)g, g_stride, M, C);
+    else if (dtype == TP_F32) mul_sigmoid_k<float><<<blocks, 256, 0, s>>>((float*)x, x_stride, (const float*)g, g_stride, M, C);
+    else return tp_fail("mul_sigmoid: unknown dtype %d", dtype);
+    return tp_check_launch("mul_sigmoid");
+}

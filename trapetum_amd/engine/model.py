@@ -94,7 +94,13 @@ class Model:
 
     def entry_state_specs(self):
         """For every schedule entry the states its block keeps beside the mixer's cache, by name."""
-        return [self.layers[e.layer].block.state_specs() for e in self.schedule]
+        out = []
+        for e in self.schedule:
+            block = self.layers[e.layer].block
+            states = dict(block.state_specs())
+            states.update({"mixer." + name: spec for name, spec in block.mixer.state_specs().items()})
+            out.append(states)
+        return out
 
     def new_cache(self, max_tokens, max_context=None, max_slots=None, page_size=64):
         max_context = max_context or max_tokens

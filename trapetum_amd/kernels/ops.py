@@ -21,9 +21,14 @@ _CORE_SIGS = {
     "tp_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "tp_latent_prepare": [_P, _L, _I, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _P],
     "tp_head_linear": [_P, _L, _L, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I, _P],
-    "tp_route_top": [_P, _I, _I, _I, _I, _P, _P, _P],
+    "tp_route_top": [_P, _I, _I, _I, _I, _I, _P, _P, _P],
     "tp_expert_ffn_workspace_bytes": [_I, _I, _I, _I, _I, _I],
-    "tp_expert_ffn": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _P, _F, _F, _F, _P, _L, _P, _I, _P],
+    "tp_expert_ffn": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _P, _F, _F, _F, _I, _P, _L, _P, _I, _P],
+    "tp_conv_act": [_P, _L, _I, _P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _P],
+    "tp_ssd_scan_workspace_bytes": [_I, _I, _I, _I, _I, _I],
+    "tp_ssd_scan": [_P, _L, _P, _L, _P, _L, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _L, _P],
+    "tp_pair_norm_mean": [_P, _P, _I, _P, _P, _F, _P, _I, _I, _P],
+    "tp_mul_sigmoid": [_P, _L, _P, _L, _I, _I, _I, _P],
     "tp_gather_rows": [_P, _P, _P, _I, _I, _I, _P],
     "tp_sum_slices": [_P, _I, _L, _P, _I, _L, _P],
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
@@ -53,7 +58,9 @@ _ATTN_SIGS = {
 
 EPI_NONE, EPI_SOFTCAP, EPI_GATED = 0, 1, 2
 ROPE_PAIRINGS = {"halves": 0, "neighbours": 1}          # the kernel library's TP_ROPE_* enumerators
-GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}       # what a gated product's epilogue can apply to the gate
+GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "relu": 2}       # what a gated product's epilogue can apply to the gate
+ROUTE_SCORES = {"softmax": 0, "sigmoid": 1}          # how a router's logits become scores
+CONV_ACTIVATIONS = {None: 0, "silu": 1}
 GATE_GROUP = 16
 
 
@@ -88,6 +95,8 @@ def _bind(lib, sigs):
 
 
 class HipOps:
+    SplitRows = SplitRows
+
     def __init__(self, device):
         if device.type != "cuda" or not torch.cuda.is_available():
             raise KernelError(
@@ -332,8 +341,11 @@ class HipOps:
         return out
 
     # ---- mixture of experts ------------------------------------------------------------------------------------
-    def route_top(self, logits, top, renormalize=False):
-        """softmax over all experts; the `top` largest scores (ties: the smaller index): int32 [M, top], float32 [M, top]."""
+    def route_top(self, logits, top, renormalize=False, score="softmax"):
+        """Scores: softmax over all experts, or the sigmoid of each logit; the `top` largest scores (ties: the smaller
+        index): int32 [M, top], float32 [M, top]."""
+        if score not in ROUTE_SCORES:
+            raise KernelError(f"route_top: score '{score}' has no kernel ({', '.join(ROUTE_SCORES)})")
         self._dev(logits)
         if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
             raise KernelError("route_top: router logits must be contiguous float32 [rows, experts]")
@@ -342,14 +354,16 @@ class HipOps:
             raise KernelError(f"route_top: {top} of {e} experts cannot be chosen")
         chosen = torch.empty((m, top), dtype=torch.int32, device=self.device)
         weight = torch.empty((m, top), dtype=torch.float32, device=self.device)
-        self._call(self.lib, "tp_route_top", logits.data_ptr(), m, e, int(top), 1 if renormalize else 0, chosen.data_ptr(),
+        self._call(self.lib, "tp_route_top", logits.data_ptr(), m, e, int(top), 1 if renormalize else 0, ROUTE_SCORES[score], chosen.data_ptr(),
                    weight.data_ptr(), self._stream())
         return chosen, weight
 
-    def expert_ffn(self, x, chosen, weights, w_gate_up, w_down, limit, alpha, shift):
+    def expert_ffn(self, x, chosen, weights, w_gate_up, w_down, limit, alpha, shift, weight_input=False, out=None):
         """float32 [M, D]: sum over a row's chosen experts of weight * W_down,e (g' sigmoid(alpha g') (u' + shift)), with
         g' = min(W_gate,e x, limit), u' = clamp(W_up,e x, -limit, limit).  w_gate_up [E, 2 F, D] (gate rows, then up
-        rows), w_down [E, D, F]."""
+        rows), w_down [E, D, F].  limit None: no clamp.  weight_input: the weight multiplies the expert's input instead,
+        expert(weight * x), and the outputs are summed as they are.  out: a contiguous float32 [M, D] to fill."""
+        limit = float("inf") if limit is None else limit
         self._dev(x, chosen, weights, w_gate_up, w_down)
         if x.dim() != 2 or not x.is_contiguous() or x.dtype != w_gate_up.dtype or x.dtype != w_down.dtype:
             raise KernelError("expert_ffn: rows and matrices must be contiguous and of one dtype")
@@ -366,11 +380,105 @@ class HipOps:
             raise KernelError("expert_ffn: the choice must be int32 [rows, top] with float32 weights of the same shape")
         nbytes = self.lib.tp_expert_ffn_workspace_bytes(_code(x.dtype), m, top, e, f, d)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
-        out = torch.empty((m, d), dtype=torch.float32, device=self.device)
+        if out is None:
+            out = torch.empty((m, d), dtype=torch.float32, device=self.device)
+        elif out.dtype != torch.float32 or tuple(out.shape) != (m, d) or not out.is_contiguous():
+            raise KernelError(f"expert_ffn: the output must be contiguous float32 {(m, d)}")
+        self._dev(out)
         self._call(self.lib, "tp_expert_ffn", x.data_ptr(), _code(x.dtype), m, d, chosen.data_ptr(), weights.data_ptr(), top, e, f,
-                   w_gate_up.data_ptr(), w_down.data_ptr(), float(limit), float(alpha), float(shift), ws.data_ptr(), nbytes,
+                   w_gate_up.data_ptr(), w_down.data_ptr(), float(limit), float(alpha), float(shift), 1 if weight_input else 0,
+                   ws.data_ptr(), nbytes,
                    out.data_ptr(), 1 if self.force_linear == 1 else 0, self._stream())
         return out
+
+    # ---- a state-space mixer; two mixers side by side ------------------------------------------------------------------
+    def conv_act(self, x, w_t, bias, state, slot_ids, cu_rows, row_seq, activation=None, one_row_each=False):
+        """out[r] = act(bias + sum_j w_t[j] * x[r - (taps - 1) + j]) within each sequence, on a view x [M, C] of wider rows;
+        the rows before the step are read from state[slot] (float32 [slots, taps - 1, C], oldest first), which then takes
+        the last taps - 1 rows of (state, step).  w_t: float32 [taps, C].  Returns a contiguous [M, C] of x's dtype."""
+        if activation not in CONV_ACTIVATIONS:
+            raise KernelError(f"conv_act: activation '{activation}' has no kernel")
+        self._dev(x, w_t, bias, state, slot_ids, cu_rows, row_seq)
+        stride = self._rows(x, "conv_act rows")
+        m, c = x.shape
+        if w_t.dtype != torch.float32 or w_t.dim() != 2 or w_t.shape[1] != c or not w_t.is_contiguous():
+            raise KernelError(f"conv_act: the taps must be contiguous float32 [taps, {c}]")
+        taps, n_seq = w_t.shape[0], cu_rows.numel() - 1
+        if bias is not None and (bias.dtype != torch.float32 or bias.numel() != c or not bias.is_contiguous()):
+            raise KernelError(f"conv_act: the bias must be contiguous float32 [{c}]")
+        for t, n in ((cu_rows, n_seq + 1), (row_seq, m), (slot_ids, n_seq)):
+            if t.dtype != torch.int32 or t.numel() != n:
+                raise KernelError("conv_act: cu_rows, row_seq and slot_ids must be int32 of the step's geometry")
+        if taps > 1 and (state is None or state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (taps - 1, c)
+                         or not state.is_contiguous()):
+            raise KernelError(f"conv_act: the state must be contiguous float32 [slots, {taps - 1}, {c}]")
+        out = torch.empty((m, c), dtype=x.dtype, device=self.device)
+        self._call(self.lib, "tp_conv_act", x.data_ptr(), stride, _code(x.dtype), w_t.data_ptr(), bias.data_ptr() if bias is not None else None,
+                   state.data_ptr() if taps > 1 else None, slot_ids.data_ptr(), cu_rows.data_ptr(), row_seq.data_ptr(), out.data_ptr(), c,
+                   _code(out.dtype), m, n_seq, c, taps, CONV_ACTIVATIONS[activation], 1 if one_row_each else 0, self._stream())
+        return out
+
+    SSD_CHUNK = 64                 # rows of a piece when a long scan is cut into pieces that run side by side
+
+    def ssd_scan(self, xbc, z, dt, dt_bias, a_log, skip, state, slot_ids, cu_rows, max_count, heads, groups, n_state, head_dim):
+        """The recurrence of a state-space mixer over the step's rows, sequence by sequence, from state[slot] (float32
+        [slots, heads, n_state, head_dim]), which it leaves updated:
+            S <- exp(-exp(a_log) d) S + d B x^T,  y = (S^T C + skip x) * silu(z),  d = softplus(dt + dt_bias)
+        xbc [M, heads head_dim + 2 groups n_state] = [x | B | C]; z [M, heads head_dim] and dt [M, heads] may be views of
+        wider rows.  Returns y float32 [M, heads head_dim]."""
+        self._dev(xbc, z, dt, dt_bias, a_log, skip, state, slot_ids, cu_rows)
+        m = xbc.shape[0]
+        inner = heads * head_dim
+        xs, zs, ds = self._rows(xbc, "ssd_scan xbc"), self._rows(z, "ssd_scan z"), self._rows(dt, "ssd_scan dt")
+        if xbc.shape[1] != inner + 2 * groups * n_state or tuple(z.shape) != (m, inner) or tuple(dt.shape) != (m, heads):
+            raise KernelError(f"ssd_scan: rows {tuple(xbc.shape)}, gates {tuple(z.shape)} and steps {tuple(dt.shape)} do not fit "
+                              f"{heads} heads of {head_dim}, {groups} groups and a state of {n_state}")
+        if not (xbc.dtype == z.dtype == dt.dtype):
+            raise KernelError("ssd_scan: rows, gates and steps share one dtype")
+        if heads % groups:
+            raise KernelError(f"ssd_scan: {heads} heads are no multiple of {groups} groups")
+        for t in (dt_bias, a_log, skip):
+            if t.dtype != torch.float32 or t.numel() != heads or not t.is_contiguous():
+                raise KernelError(f"ssd_scan: dt_bias, a_log and skip must be contiguous float32 [{heads}]")
+        n_seq = cu_rows.numel() - 1
+        if slot_ids.dtype != torch.int32 or slot_ids.numel() != n_seq or cu_rows.dtype != torch.int32:
+            raise KernelError("ssd_scan: slot_ids and cu_rows must be int32 of the step's geometry")
+        if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, n_state, head_dim) or not state.is_contiguous():
+            raise KernelError(f"ssd_scan: the state must be contiguous float32 [slots, {heads}, {n_state}, {head_dim}]")
+        y = torch.empty((m, inner), dtype=torch.float32, device=self.device)
+        # pieces enough to give the GPU some four thousand waves, of at least SSD_CHUNK rows each
+        waves = n_seq * heads * -(-head_dim // 64)
+        chunk = max(self.SSD_CHUNK, -(-int(max_count) // max(1, 4096 // waves)))
+        chunk = -(-chunk // 16) * 16
+        nbytes = self.lib.tp_ssd_scan_workspace_bytes(n_seq, int(max_count), heads, n_state, head_dim, chunk)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device) if nbytes else None
+        self._call(self.lib, "tp_ssd_scan", xbc.data_ptr(), xs, z.data_ptr(), zs, dt.data_ptr(), ds, _code(xbc.dtype), dt_bias.data_ptr(),
+                   a_log.data_ptr(), skip.data_ptr(), state.data_ptr(), slot_ids.data_ptr(), cu_rows.data_ptr(), y.data_ptr(), n_seq,
+                   int(max_count), heads, groups, n_state, head_dim, chunk, ws.data_ptr() if ws is not None else None, nbytes, self._stream())
+        return y
+
+    def pair_norm_mean(self, a, b, gain_a, gain_b, eps):
+        """float32 [M, D]: 0.5 (a / rms(a) * gain_a + b / rms(b) * gain_b), each row over its own root mean square."""
+        self._dev(a, b, gain_a, gain_b)
+        if a.dim() != 2 or a.shape != b.shape or a.dtype != b.dtype or not a.is_contiguous() or not b.is_contiguous():
+            raise KernelError("pair_norm_mean: two contiguous matrices of one shape and dtype")
+        m, d = a.shape
+        for g in (gain_a, gain_b):
+            if g.dtype != torch.float32 or g.numel() != d or not g.is_contiguous():
+                raise KernelError(f"pair_norm_mean: gains must be contiguous float32 [{d}]")
+        out = torch.empty((m, d), dtype=torch.float32, device=self.device)
+        self._call(self.lib, "tp_pair_norm_mean", a.data_ptr(), b.data_ptr(), _code(a.dtype), gain_a.data_ptr(), gain_b.data_ptr(), float(eps),
+                   out.data_ptr(), m, d, self._stream())
+        return out
+
+    def mul_sigmoid(self, x, g):
+        """x *= sigmoid(g), in place; both [M, C] of one dtype, possibly views of wider rows."""
+        self._dev(x, g)
+        xs, gs = self._rows(x, "mul_sigmoid rows"), self._rows(g, "mul_sigmoid gates")
+        if x.shape != g.shape or x.dtype != g.dtype:
+            raise KernelError("mul_sigmoid: rows and gates of one shape and dtype")
+        self._call(self.lib, "tp_mul_sigmoid", x.data_ptr(), xs, g.data_ptr(), gs, _code(x.dtype), x.shape[0], x.shape[1], self._stream())
+        return x
 
     MAX_SLICED_WIDTH = 8192        # widest row `add_rms_norm` takes in K slices
 
@@ -449,7 +557,7 @@ class HipOps:
                    v_pool.data_ptr(), k_pool.shape[2], rows_cap, self._stream())
 
     # ---- matrix products -----------------------------------------------------------------------------
-    def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False, act=0):
+    def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False, act=0, out=None):
         self._dev(x, w)
         if x.dim() != 2 or w.dim() != 2 or not x.is_contiguous() or not w.is_contiguous():
             raise KernelError("linear: rows and matrix must be contiguous 2-D tensors")
@@ -468,17 +576,26 @@ class HipOps:
             self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), None, _code(x.dtype), _code(out_dtype),
                        m, n, k, epilogue, float(cap), units, act, slices.data_ptr(), nbytes, 1, algo, self._stream())
             return SplitRows(slices)
-        out = torch.empty((m, cols), dtype=out_dtype, device=self.device)
+        if out is None:
+            out = torch.empty((m, cols), dtype=out_dtype, device=self.device)
+        elif out.dtype != out_dtype or tuple(out.shape) != (m, cols) or not out.is_contiguous():
+            raise KernelError(f"linear: the output must be contiguous {out_dtype} {(m, cols)}")
+        self._dev(out)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device) if nbytes else None
         self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(x.dtype), _code(out_dtype),
                    m, n, k, epilogue, float(cap), units, act, ws.data_ptr() if ws is not None else None, nbytes, 0, algo,
                    self._stream())
         return out
 
-    def linear(self, x, w, out_dtype, softcap=None, defer=False, bias=None):
+    def linear(self, x, w, out_dtype, softcap=None, defer=False, bias=None, out=None):
         """x @ w^T (+ bias).  defer: the caller hands the result to `add_rms_norm` (or through `rows()`), so a product
         computed in K slices may come back as SplitRows.  bias: float32 [rows of w], added by a kernel of its own
-        (the products have no bias operand), so a product with a bias is never left in slices."""
+        (the products have no bias operand), so a product with a bias is never left in slices.  out: a contiguous
+        tensor to fill (a plain product only)."""
+        if out is not None:
+            if bias is not None or softcap or defer:
+                raise KernelError("linear: an output to fill goes with a plain product only")
+            return self._linear(x, w, out_dtype, EPI_NONE, 0.0, 0, out=out)
         if bias is not None:
             if softcap:
                 raise KernelError("linear: a bias and a cap together have no kernel")

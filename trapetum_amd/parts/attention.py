@@ -10,7 +10,10 @@ reference fixes the scale to rsqrt(head_dim) (cu:249) and has no window
 t <= p, and with a window W only those with p - t < W.
 
 The three projections are one product over the concatenated weight.  A run that
-reads another run's cache projects and rotates its queries only.  In a decode step
+reads another run's cache projects and rotates its queries only (a layer may also have no key and value
+projections at all, `own_kv=False`).  Values may have another size than keys (`value_dim`), the heads' outputs
+may pass a sigmoid gate computed from the layer's input (`output_gate`), and a position scheme that turns
+neighbouring elements is carried out as the rotation of halves on reordered projection rows.  In a decode step
 rotation, cache write and attention are one kernel launch where the kernel library
 has one for the geometry (`ops.fuses_decode_step`); the order of the arithmetic is
 the same.  A step that continues sequences by several tokens, or mixes starting and running sequences, attends
@@ -26,74 +29,125 @@ from .base import Mixer
 
 class Attention(Mixer):
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, query_scale,
-                 softcap=None, window=None, position=("none", {})):
+                 softcap=None, window=None, position=("none", {}), value_dim=None, output_gate=False, own_kv=True,
+                 tensors=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight", "g_proj.weight")):
+        """value_dim: elements of a value head when they differ from a key's head_dim.  output_gate: the heads' outputs
+        are multiplied by sigmoid(W_g x) before the output projection.  own_kv False: the layer has no key and value
+        projections; its schedule entry names the run whose cache it reads.  tensors: local names of W_q, W_k, W_v, W_o
+        (and W_g)."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} kv heads")
         self.hidden_size = hidden_size
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads
         self.head_dim = head_dim
+        self.value_dim = int(value_dim) if value_dim else head_dim
+        # The kernels know one head size: keys and values are kept in rows of the larger of the two, the shorter kind
+        # filled up with zeros through zero rows of its projection (zeros add nothing to a score, and a value's zero
+        # columns meet zero columns of W_o).
+        self.row = max(self.head_dim, self.value_dim)
         self.query_scale = float(query_scale)
         self.softcap = float(softcap) if softcap else 0.0
         self.window = int(window) if window else 0
+        self.output_gate = bool(output_gate)
+        self.own_kv = bool(own_kv)
+        self.names = dict(zip(("q", "k", "v", "o", "g"), tuple(tensors) + ("g_proj.weight",) * (5 - len(tensors))))
         self.position = build_part("position", position)
         if self.position.rotary_dim > head_dim:
             raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head_dim {head_dim}")
 
     def tensor_specs(self):
-        d, q, kv = self.hidden_size, self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
-        return {"q_proj.weight": TensorSpec((q, d)), "k_proj.weight": TensorSpec((kv, d)),
-                "v_proj.weight": TensorSpec((kv, d)), "o_proj.weight": TensorSpec((d, q))}
+        n, d = self.names, self.hidden_size
+        q, kv = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        specs = {n["q"]: TensorSpec((q, d)), n["o"]: TensorSpec((d, self.num_heads * self.value_dim))}
+        if self.own_kv:
+            specs[n["k"]] = TensorSpec((kv, d))
+            specs[n["v"]] = TensorSpec((self.num_kv_heads * self.value_dim, d))
+        if self.output_gate:
+            specs[n["g"]] = TensorSpec((self.num_heads * self.value_dim, d))
+        return specs
 
     def cache_spec(self):
-        per_token = (self.num_kv_heads, self.head_dim)
+        per_token = (self.num_kv_heads, self.row)
         return TokenSpec.of(self.window or None, k=per_token, v=per_token)
+
+    def _heads(self, w, heads, size, turned=False):
+        """[heads * size, d] -> [heads * row, d]: zero rows fill a head up to `row`.  turned: a rotation of neighbouring
+        pairs (2f, 2f + 1) becomes the rotation of halves (f, f + rotary_dim / 2) that every kernel knows by taking
+        a head's even rotated rows first, then its odd ones; queries and keys are reordered alike, so every score is
+        the same sum in another order."""
+        import torch
+        w = w.reshape(heads, size, -1)
+        rot = self.position.rotary_dim
+        if turned and rot and self.position.pairing == "neighbours":
+            order = list(range(0, rot, 2)) + list(range(1, rot, 2)) + list(range(rot, size))
+            w = w[:, order]
+        if size < self.row:
+            w = torch.cat([w, w.new_zeros((heads, self.row - size, w.shape[2]))], dim=1)
+        return w.reshape(heads * self.row, -1)
 
     def bind(self, tensors, rt):
         import torch
         self.rt = rt
-        self.w_qkv = rt.matrix(torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
-                                          tensors["v_proj.weight"]], dim=0)).contiguous()
-        self.w_o = rt.matrix(tensors["o_proj.weight"])
+        n, H, KV = self.names, self.num_heads, self.num_kv_heads
+        parts = [self._heads(tensors[n["q"]], H, self.head_dim, turned=True)]
+        if self.own_kv:
+            parts += [self._heads(tensors[n["k"]], KV, self.head_dim, turned=True), self._heads(tensors[n["v"]], KV, self.value_dim)]
+        self.w_qkv = rt.matrix(torch.cat(parts, dim=0)).contiguous()
+        self.w_g = rt.matrix(self._heads(tensors[n["g"]], H, self.value_dim).contiguous()) if self.output_gate else None
+        w_o = tensors[n["o"]]
+        if self.value_dim < self.row:
+            w_o = torch.cat([w_o.reshape(-1, H, self.value_dim), w_o.new_zeros((w_o.shape[0], H, self.row - self.value_dim))], dim=2)
+            w_o = w_o.reshape(-1, H * self.row).contiguous()
+        self.w_o = rt.matrix(w_o)
         self.inv_freq = self.position.inv_freq(rt.device)
+
+    def _project_out(self, ctx, x, out):
+        if self.output_gate:
+            ctx.ops.mul_sigmoid(out, ctx.ops.linear(x, self.w_g, ctx.dtype))
+        return ctx.ops.linear(out, self.w_o, ctx.dtype, defer=True)
 
     def forward(self, ctx, x, site):
         ops = ctx.ops
-        H, KV, hd = self.num_heads, self.num_kv_heads, self.head_dim
+        H, KV, hd = self.num_heads, self.num_kv_heads, self.row
         Q, KVD = H * hd, KV * hd
         owns_cache = ctx.cache_owner == ctx.entry
+        if owns_cache and not self.own_kv:
+            raise ValueError("an attention without key and value projections must read another run's cache")
+        w_in = self.w_qkv if owns_cache else self.w_qkv[:Q]          # a run on another run's cache projects its queries only
         if site.spec.window is not None and not 0 < self.window <= site.spec.window:
             raise ValueError(f"this attention sees {self.window or 'all'} keys back, the cache it reads keeps {site.spec.window}")
+        if site.spec.shape_of("k") != (KV, hd):
+            raise ValueError(f"the cache read here keeps keys of {site.spec.shape_of('k')}, this layer needs {(KV, hd)}")
         table = ctx.page_table(site.group_index)
-        k_pool, v_pool = site.tensor("k"), site.tensor("v")         # [pages, kv_heads, page, head_dim]
+        k_pool, v_pool = site.tensor("k"), site.tensor("v")         # [pages, kv_heads, page, row]
         rows_cap = site.rows_cap or 0
-        pairing = self.position.pairing
-        if ctx.mode == "decode" and pairing == "halves" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, k_pool):
+        if ctx.mode == "decode" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, k_pool):
             # one launch rotates, writes the cache and attends; the projections may stay in K slices until then
-            qkv = ops.linear(x, self.w_qkv if owns_cache else self.w_qkv[:Q], ctx.dtype, defer=True)
+            qkv = ops.linear(x, w_in, ctx.dtype, defer=True)
             out = ops.attention_decode_step(qkv, H, KV, hd, self.inv_freq, self.position.rotary_dim, ctx.new_len,
                                             table, k_pool, v_pool, rows_cap, self.query_scale, self.softcap,
                                             self.window, ctx.dtype, max_keys=ctx.max_rows_visible(site), write_kv=owns_cache)
-            return ops.linear(out, self.w_o, ctx.dtype, defer=True)
+            return self._project_out(ctx, x, out)
+        qkv = ops.linear(x, w_in, ctx.dtype)
         if owns_cache:
-            qkv = ops.linear(x, self.w_qkv, ctx.dtype)
             q, k, v = qkv[:, :Q], qkv[:, Q:Q + KVD], qkv[:, Q + KVD:]
         else:
-            q, k, v = ops.linear(x, self.w_qkv[:Q], ctx.dtype), None, None
+            q, k, v = qkv, None, None
         if ctx.mode == "decode":
             ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
-                              ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap, pairing=pairing)
+                              ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap)
             out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, k_pool, v_pool, rows_cap,
                                        self.query_scale, self.softcap, self.window, ctx.dtype,
                                        max_keys=ctx.max_rows_visible(site))
-            return ops.linear(out, self.w_o, ctx.dtype, defer=True)
+            return self._project_out(ctx, x, out)
         # Sequences that go on by several tokens (or some start while others go on) see cached positions and the
         # step's own rows.  The attention reads the cached ones where they lie, as earlier steps left them, and the
         # step's rows from the step; only then are the step's rows cached: in a window's ring without a row to spare
         # they take the places of positions that the step's earlier queries still see.
         extend = ctx.mode == "extend"
         ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
-                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap, pairing=pairing,
+                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap,
                           write=not extend)
         if owns_cache:
             ctx.offer_step_rows(k=k, v=v)
@@ -107,7 +161,7 @@ class Attention(Mixer):
         if extend and owns_cache:
             row_seq, row_pos, new_len = ctx.row_seq, ctx.row_pos, ctx.new_len
             ctx.after_readers(lambda: ops.kv_write(k, v, KV, hd, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap))
-        return ops.linear(out, self.w_o, ctx.dtype, defer=True)
+        return self._project_out(ctx, x, out)
 
 
 register_part("mixer", "attention", Attention)

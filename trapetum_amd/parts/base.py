@@ -8,7 +8,8 @@ step (`forward`).  Interfaces:
                norm multiplies by, so that blocks can fuse a norm into a neighbour.
   Position     `rotary_dim` and `inv_freq(device)`: the rotation table a mixer applies
                to queries and keys before the cache write.
-  Mixer        cache_spec() -> TokenSpec | StateSpec | None;
+  Mixer        cache_spec() -> TokenSpec | StateSpec | None;  state_specs() -> {name: StateSpec} of further states
+               (`self.state(ctx, name)`), so that one mixer may keep tensors per token and states, or hold other mixers;
                forward(ctx, x, site) -> rows [M, hidden], x being the normed rows.
   FeedForward  forward(ctx, x) -> rows [M, hidden].
                (A mixer or feed-forward may return what `ops.linear(..., defer=True)` gave it: the block
@@ -56,8 +57,19 @@ class Position(Part):
 
 
 class Mixer(Part):
+    state_scope = ""          # set by a mixer that holds this one: the prefix of its states' names
+
     def cache_spec(self):
         return None
+
+    def state_specs(self):
+        """{name: StateSpec} of what the mixer keeps per sequence beside its cache_spec (a mixer that keeps tensors per
+        token and states, or several states)."""
+        return {}
+
+    def state(self, ctx, name):
+        """The running entry's state `name` of this mixer: [slots + 1, *shape]."""
+        return ctx.cache.entry_state(ctx.entry, "mixer." + self.state_scope + name)
 
     def forward(self, ctx, x, site):
         raise NotImplementedError

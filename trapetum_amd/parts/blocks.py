@@ -36,6 +36,12 @@ def add_then_norm(ctx, stream, rows, post, nxt):
 
 
 class SandwichBlock(Block):
+    def __init__(self, mixer, feed_forward, make_norm):
+        self.mixer = mixer
+        self.feed_forward = feed_forward                 # None: the layer is its mixer, with the norms around it
+        sites = self.norm_sites() if feed_forward is not None else self.norm_sites()[:2]
+        self.norms = {name: make_norm(name) for name in sites}
+
     @classmethod
     def norm_sites(cls):
         return ("pre_mixer_norm", "post_mixer_norm", "pre_ff_norm", "post_ff_norm")
@@ -49,6 +55,10 @@ class SandwichBlock(Block):
         ctx.dump("mixer_in", x)
         a = self.mixer.forward(ctx, x, site)
         ctx.dump("mixer_out", a)
+        if self.feed_forward is None:
+            normed_next = add_then_norm(ctx, stream, a, n["post_mixer_norm"], next_norm)
+            ctx.dump("layer_out", stream)
+            return stream, normed_next
         x = add_then_norm(ctx, stream, a, n["post_mixer_norm"], n["pre_ff_norm"])
         ctx.dump("after_mixer", stream)
         m = self.feed_forward.forward(ctx, x)

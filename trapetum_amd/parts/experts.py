@@ -13,14 +13,30 @@ from .base import FeedForward
 
 class RoutedExperts(FeedForward):
     def __init__(self, hidden_size, intermediate_size, n_experts, top, limit, gate_alpha=1.702, up_shift=1.0,
-                 renormalize=False, router="router", expert="e{}.", tensors=("gate", "up", "down")):
+                 renormalize=False, router="router", expert="e{}.", tensors=("gate", "up", "down"),
+                 score="softmax", weight_input=False, shared=None):
+        """limit None: gate and up sums are not clamped (with gate_alpha 1 and up_shift 0 the expert is SiLU-gated).
+        score: "softmax" over all experts or the "sigmoid" of each logit.  weight_input: a chosen expert's score
+        multiplies its input, expert(s h), instead of its output.  shared: (registered feed-forward, parameters) of a
+        layer that every token passes as well; its output is added."""
         if not 0 < top <= n_experts:
             raise ValueError(f"{top} of {n_experts} experts cannot be chosen")
+        if score not in ("softmax", "sigmoid"):
+            raise ValueError(f"a router's scores are softmax or sigmoid, not '{score}'")
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.n_experts, self.top = int(n_experts), int(top)
-        self.limit, self.gate_alpha, self.up_shift = float(limit), float(gate_alpha), float(up_shift)
+        self.limit = None if limit is None else float(limit)
+        self.gate_alpha, self.up_shift = float(gate_alpha), float(up_shift)
         self.renormalize = bool(renormalize)
+        self.score, self.weight_input = score, bool(weight_input)
         self.router_name, self.expert_name, self.names = router, expert, tuple(tensors)
+        self.shared, self.shared_prefix = None, ""
+        if shared is not None:
+            from ..registry import build_part
+            name, params = shared
+            params = dict(params)
+            self.shared_prefix = params.pop("prefix", "shared.")
+            self.shared = build_part("feed_forward", (name, params))
 
     def tensor_specs(self):
         d, i = self.hidden_size, self.intermediate_size
@@ -29,6 +45,8 @@ class RoutedExperts(FeedForward):
         for e in range(self.n_experts):
             p = self.expert_name.format(e)
             specs.update({p + g: TensorSpec((i, d)), p + u: TensorSpec((i, d)), p + dn: TensorSpec((d, i))})
+        if self.shared is not None:
+            specs.update({self.shared_prefix + k: v for k, v in self.shared.tensor_specs().items()})
         return specs
 
     def bind(self, tensors, rt):
@@ -40,13 +58,23 @@ class RoutedExperts(FeedForward):
         # [experts, 2 ff, width]: an expert's gate rows, then its up rows; [experts, width, ff]
         self.w_gate_up = rt.matrix(torch.stack([torch.cat([tensors[p + g], tensors[p + u]], dim=0) for p in ex]).contiguous())
         self.w_down = rt.matrix(torch.stack([tensors[p + dn] for p in ex]).contiguous())
+        if self.shared is not None:
+            self.shared.bind({k: tensors[self.shared_prefix + k] for k in self.shared.tensor_specs()}, rt)
 
     def forward(self, ctx, x):
         import torch
         ops = ctx.ops
         logits = ops.linear(x, self.w_router, torch.float32)        # fp32 sums of exact products
-        chosen, weights = ops.route_top(logits, self.top, self.renormalize)
-        return ops.expert_ffn(x, chosen, weights, self.w_gate_up, self.w_down, self.limit, self.gate_alpha, self.up_shift)
+        chosen, weights = ops.route_top(logits, self.top, self.renormalize, score=self.score)
+        if self.shared is None:
+            return ops.expert_ffn(x, chosen, weights, self.w_gate_up, self.w_down, self.limit, self.gate_alpha, self.up_shift,
+                                  weight_input=self.weight_input)
+        # the experts' sum and the shared layer's output as two slices that the block's add forms the sum of
+        both = torch.empty((2, x.shape[0], self.hidden_size), dtype=torch.float32, device=x.device)
+        ops.expert_ffn(x, chosen, weights, self.w_gate_up, self.w_down, self.limit, self.gate_alpha, self.up_shift,
+                       weight_input=self.weight_input, out=both[0])
+        self.shared.forward(ctx, x, out=both[1])
+        return ops.SplitRows(both)
 
 
 register_part("feed_forward", "routed_experts", RoutedExperts)

@@ -30,8 +30,11 @@ class GatedMLP(FeedForward):
         self.w_gate_up = rt.ops.pack_gate_up(rt.matrix(tensors[g]), rt.matrix(tensors[u]))
         self.w_down = rt.matrix(tensors[dn])
 
-    def forward(self, ctx, x):
+    def forward(self, ctx, x, out=None):
+        """out: a contiguous float32 [M, hidden] to fill (a caller that adds this layer's output to another's)."""
         act = ctx.ops.gated_linear(x, self.w_gate_up, self.intermediate_size, self.activation, ctx.dtype)
+        if out is not None:
+            return ctx.ops.linear(act, self.w_down, out.dtype, out=out)
         return ctx.ops.linear(act, self.w_down, ctx.dtype, defer=True)
 
 

@@ -10,6 +10,8 @@ how the reference carries its scaled variants too (runtime/src/lib.rs:1071-1076)
 or "neighbours" (2d, 2d + 1); the kernel that fuses a decode step's rotation with its
 attention knows the halves only, so another pairing takes the separate launches.
 """
+import math
+
 import torch
 
 from ..registry import register_part
@@ -17,7 +19,10 @@ from .base import Position
 
 
 class RotaryPosition(Position):
-    def __init__(self, rotary_dim, theta, pairing="halves"):
+    def __init__(self, rotary_dim, theta, pairing="halves", scaling=None):
+        """scaling: None, or {"factor", "low", "high", "original"}: a frequency f whose wavelength 2 pi / f is longer than
+        original / low is divided by factor, one shorter than original / high is kept, and in between the two are mixed,
+        (1 - s) f / factor + s f with s = (original / wavelength - low) / (high - low)."""
         if rotary_dim % 2:
             raise ValueError(f"rotary_dim {rotary_dim} must be even")
         if pairing not in ("halves", "neighbours"):
@@ -25,13 +30,26 @@ class RotaryPosition(Position):
         self.rotary_dim = rotary_dim
         self.theta = float(theta)
         self.pairing = pairing
+        self.scaling = None
+        if scaling is not None:
+            self.scaling = {k: float(scaling[k]) for k in ("factor", "low", "high", "original")}
+            if self.scaling["high"] <= self.scaling["low"] or self.scaling["factor"] <= 0:
+                raise ValueError(f"frequency scaling {scaling!r}: high must exceed low and factor be positive")
         self._tables = {}
 
     def inv_freq(self, device):
         key = str(device)
         if key not in self._tables:
             e = torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / self.rotary_dim
-            self._tables[key] = (1.0 / (self.theta ** e)).to(device)
+            f = 1.0 / (self.theta ** e)
+            if self.scaling is not None:
+                sc = self.scaling
+                wave = 2.0 * math.pi / f
+                s = ((sc["original"] / wave - sc["low"]) / (sc["high"] - sc["low"])).clamp(0.0, 1.0)
+                mixed = (1.0 - s) * f / sc["factor"] + s * f
+                f = torch.where(wave > sc["original"] / sc["low"], f / sc["factor"],
+                                torch.where(wave < sc["original"] / sc["high"], f, mixed))
+            self._tables[key] = f.to(torch.float32).to(device)
         return self._tables[key]
 
 
