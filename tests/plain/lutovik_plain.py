@@ -231,3 +231,13 @@ def forward(cfg, t, tokens, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return norm_one_plus(x, t["final.norm"], eps) @ t["head"].T
+
+
+def greedy_generate(cfg, t, prompt, n):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        z = forward(cfg, t, toks)[-1]
+        tok = int(torch.nonzero(z == z.max())[0])
+        out.append(tok)
+        toks.append(tok)
+    return out

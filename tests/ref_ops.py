@@ -155,7 +155,7 @@ def gated_linear(x, w_packed, inter, activation, out_dtype):
 def _rotate(x, pos, inv_freq, rotary_dim, pairing="halves"):
     """x [M, heads, hd] fp32, pos [M]."""
     if inv_freq is None or rotary_dim == 0:
-        return x
+        return x.clone()
     half = rotary_dim // 2
     ang = pos.float()[:, None] * inv_freq[None, :]
     c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]

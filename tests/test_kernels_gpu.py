@@ -219,14 +219,16 @@ def test_gated_linear(ops, algo, dt, m, inter, k):
     try:
         got = ops.gated_linear(x, packed, inter, "gelu_tanh", DT[dt])
         silu = ops.gated_linear(x, packed, inter, "silu", DT[dt])
+        relu = ops.gated_linear(x, packed, inter, "relu", DT[dt])
         with pytest.raises(Exception, match="no kernel"):
-            ops.gated_linear(x, packed, inter, "relu", DT[dt])
+            ops.gated_linear(x, packed, inter, "softsign", DT[dt])
     finally:
         ops.force_linear = 0
     g, u = x.cpu().double() @ wg.cpu().double().T, x.cpu().double() @ wu.cpu().double().T
     ref = torch.nn.functional.gelu(g, approximate="tanh") * u
     assert rel_l2(got, ref) < (5e-6 if dt == "f32" else 4e-3)
-    assert rel_l2(silu, torch.nn.functional.silu(g) * u) < (5e-6 if dt == "f32" else 4e-3)      # the other activation offered
+    assert rel_l2(silu, torch.nn.functional.silu(g) * u) < (5e-6 if dt == "f32" else 4e-3)      # the other activations offered
+    assert rel_l2(relu, torch.relu(g) * u) < (5e-6 if dt == "f32" else 4e-3)
 
 
 @pytest.mark.parametrize("algo,m", [(2, 8), (3, 8), (3, 200), (5, 8), (5, 3)])
