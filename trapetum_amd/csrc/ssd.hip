@@ -36,6 +36,60 @@ conv_act_k(const TI* __restrict__ x, long x_stride, const float* __restrict__ wt
     }
 }
 
+// VEC neighbouring elements of T as one load or store
+template <typename T, int VEC> struct alignas(sizeof(T) * VEC) Pack { T v[VEC]; };
+
+// The same for channel counts and strides in whole packs of VEC: a thread takes VEC neighbouring channels.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+conv_act_vec_k(const T* __restrict__ x, long x_stride, const float* __restrict__ wt, const float* __restrict__ bias,
+               float* __restrict__ state, const int* __restrict__ slot_ids, const int* __restrict__ cu_rows,
+               const int* __restrict__ row_seq, T* __restrict__ out, long out_stride, int C, int taps, int act, int one_row_each) {
+    using P = Pack<T, VEC>;
+    using PF = Pack<float, VEC>;
+    const int r = blockIdx.x, c = (blockIdx.y * 256 + threadIdx.x) * VEC;
+    if (c >= C) return;
+    const int seq = row_seq[r], i = r - cu_rows[seq], S = taps - 1;
+    float* st = S > 0 ? state + (size_t)slot_ids[seq] * S * C + c : nullptr;
+    const P xr = *reinterpret_cast<const P*>(x + (size_t)r * x_stride + c);
+    float acc[VEC];
+    if (bias) {
+        const PF b = *reinterpret_cast<const PF*>(bias + c);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = b.v[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = 0.f;
+    }
+    for (int j = 0; j < taps; j++) {
+        const int src = i - (S - j);
+        const PF w = *reinterpret_cast<const PF*>(wt + (size_t)j * C + c);
+        if (j == S || src >= 0) {
+            const P v = j == S ? xr : *reinterpret_cast<const P*>(x + (size_t)(r - (S - j)) * x_stride + c);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) acc[e] = __builtin_fmaf(w.v[e], ld_f32(&v.v[e]), acc[e]);
+        } else {
+            const PF v = *reinterpret_cast<const PF*>(st + (size_t)(S + src) * C);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) acc[e] = __builtin_fmaf(w.v[e], v.v[e], acc[e]);
+        }
+    }
+    P o;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        const float v = act == TP_CONV_ACT_SILU ? acc[e] / (1.f + expf(-acc[e])) : acc[e];
+        st_f32(&o.v[e], v);
+    }
+    *reinterpret_cast<P*>(out + (size_t)r * out_stride + c) = o;
+    if (one_row_each && S > 0) {
+        for (int s = 0; s + 1 < S; s++) *reinterpret_cast<PF*>(st + (size_t)s * C) = *reinterpret_cast<const PF*>(st + (size_t)(s + 1) * C);
+        PF last;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) last.v[e] = ld_f32(&xr.v[e]);
+        *reinterpret_cast<PF*>(st + (size_t)(S - 1) * C) = last;
+    }
+}
+
 // grid (sequences, channel blocks): the state takes the last taps - 1 rows of (state, the step's rows)
 template <typename TI>
 __global__ void __launch_bounds__(256)
@@ -62,7 +116,16 @@ extern "C" int tp_conv_act(const void* x, long x_stride, int in_dtype, const flo
     TP_REQUIRE(in_dtype == out_dtype && (in_dtype == TP_BF16 || in_dtype == TP_F32), "conv_act: rows and output share one dtype, bfloat16 or float32");
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(M, tp_cdiv(C, 256));
-    if (in_dtype == TP_BF16)
+    const int vec = in_dtype == TP_BF16 ? 8 : 4;         // 16 bytes of the rows a thread
+    const bool packs = C % vec == 0 && x_stride % vec == 0 && out_stride % vec == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+                       (uintptr_t)wt % 32 == 0 && (!bias || (uintptr_t)bias % 32 == 0) && (!state || (uintptr_t)state % 32 == 0);
+    if (packs) {
+        dim3 vgrid(M, tp_cdiv(C / vec, 256));
+        if (in_dtype == TP_BF16)
+            conv_act_vec_k<bf16_t, 8><<<vgrid, 256, 0, s>>>((const bf16_t*)x, x_stride, wt, bias, state, slot_ids, cu_rows, row_seq, (bf16_t*)out, out_stride, C, taps, act, one_row_each);
+        else
+            conv_act_vec_k<float, 4><<<vgrid, 256, 0, s>>>((const float*)x, x_stride, wt, bias, state, slot_ids, cu_rows, row_seq, (float*)out, out_stride, C, taps, act, one_row_each);
+    } else if (in_dtype == TP_BF16)
         conv_act_k<bf16_t, bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)x, x_stride, wt, bias, state, slot_ids, cu_rows, row_seq, (bf16_t*)out, out_stride, C, taps, act, one_row_each);
     else
         conv_act_k<float, float><<<grid, 256, 0, s>>>((const float*)x, x_stride, wt, bias, state, slot_ids, cu_rows, row_seq, (float*)out, out_stride, C, taps, act, one_row_each);
@@ -94,19 +157,23 @@ struct SsdArgs {
 
 __device__ __forceinline__ float softplus_f(float v) { return log1pf(expf(-fabsf(v))) + fmaxf(v, 0.f); }
 
-// One wave owns 64 value channels of one head of one sequence (or of one piece of it): lane p keeps column p of the
-// state, NR elements, in registers; the rows' B and C vectors, step sizes, decays, inputs and gates are staged in LDS
-// TC rows at a time (every load of a round is asked for at once), and a row then costs the lane 2 N multiply-adds
-// with no traffic between lanes.  FULL: N == NR, no bounds in the inner loop.
+// A block of four waves owns 64 value channels of one head of one sequence (or of one piece of it): wave q keeps a
+// quarter of the state's rows, lane p column p of them, NR / 4 elements in registers, so that several blocks fit a
+// SIMD and one's waits are another's work.  The rows' B and C vectors, step sizes, decays, inputs and gates are staged
+// in LDS TC rows at a time (every load of a round is asked for at once); a row then costs a lane 3 N / 4 vector
+// instructions, and the four waves' parts of y meet in LDS once a round.  FULL: N == NR, no bounds in the inner loop.
+// VEC: elements of B and C a load takes.
 // MODE 0: the whole scan from the slot's state, which it leaves updated.
 // MODE 1: a piece (not the last) from a zero state: writes the state it ends with and its total decay, no outputs.
 // MODE 2: a piece from the state `carry` holds for its start: writes outputs; the last piece leaves the slot's state.
-template <typename T, int NR, int MODE, bool FULL>
-__global__ void __launch_bounds__(64)
+template <typename T, int NR, int MODE, bool FULL, int VEC>
+__global__ void __launch_bounds__(256)
 ssd_scan_k(SsdArgs a) {
-    constexpr int TC = 16;
-    extern __shared__ float lds[];                       // B [TC][N], C [TC][N], dt [TC], decay [TC], x [TC][64], z [TC][64]
-    const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    constexpr int TC = 16, NQ = NR / 4;
+    constexpr int J = (TC * NR / VEC + 255) / 256;       // packs of B (and of C) a thread stages a round
+    using Pk = Pack<T, VEC>;
+    extern __shared__ float lds[];                       // B [TC][N], C [TC][N], dt [TC], decay [TC], x [TC][64], z [TC][64], parts [4][TC][64]
+    const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
     const int pieces_z = MODE == 0 ? 1 : a.max_chunks;
     const int piece = MODE == 0 ? 0 : blockIdx.z % pieces_z, pc = MODE == 0 ? blockIdx.z : blockIdx.z / pieces_z;
     const int p = pc * 64 + lane;
@@ -122,52 +189,85 @@ ssd_scan_k(SsdArgs a) {
     const bool last_piece = MODE == 0 || r1 == first + count;
     if (MODE == 1 && last_piece) return;                 // nobody starts from the state the last piece ends with
     float* Bs = lds; float* Cs = lds + TC * N; float* dts = Cs + TC * N; float* dec = dts + TC;
-    float* xs = dec + TC; float* zs = xs + TC * 64;
+    float* xs = dec + TC; float* zs = xs + TC * 64; float* parts = zs + TC * 64;
     const float rate = expf(a.a_log[head]), bias = a.dt_bias[head], skip = a.skip[head];
-    float S[NR];
+    const int n0 = q * NQ;                               // the wave's rows of the state
+    float S[NQ];
     float* slot_state = a.state + (((size_t)a.slot_ids[seq] * a.heads + head) * N) * P + p;
     const float* from = slot_state;
     if (MODE == 2) from = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
 #pragma unroll
-    for (int n = 0; n < NR; n++) S[n] = (MODE != 1 && live && (FULL || n < N)) ? from[(size_t)n * P] : 0.f;
+    for (int n = 0; n < NQ; n++) S[n] = (MODE != 1 && live && (FULL || n0 + n < N)) ? from[(size_t)(n0 + n) * P] : 0.f;
     float total = 1.f;
     const size_t inner = (size_t)a.heads * P;
+    const int pl = live ? p : 0;
     for (int t0 = r0; t0 < r1; t0 += TC) {
         const int tn = min(TC, r1 - t0);
-        __syncthreads();
-        for (int i = lane; i < tn * N; i += 64) {
-            const int t = i / N, n = i - t * N;
-            const T* row = (const T*)a.xbc + (size_t)(t0 + t) * a.xbc_stride + inner + (size_t)g * N + n;
-            Bs[i] = ld_f32(row);
-            Cs[i] = ld_f32(row + (size_t)a.groups * N);
+        // every load of the round is asked for before the first is used (loads past the round's end read its last row,
+        // from an address that exists, and are dropped): a round waits for memory once
+        const int per_row = N / VEC, packs = tn * per_row;
+        Pk rb[J], rc[J];
+        T rx[TC / 4], rz[TC / 4];
+#pragma unroll
+        for (int j = 0; j < J; j++) {
+            const int c = min(tid + 256 * j, packs - 1), t = c / per_row, k = c - t * per_row;
+            const T* row = (const T*)a.xbc + (size_t)(t0 + t) * a.xbc_stride + inner + (size_t)g * N + k * VEC;
+            rb[j] = *reinterpret_cast<const Pk*>(row);
+            rc[j] = *reinterpret_cast<const Pk*>(row + (size_t)a.groups * N);
         }
-        for (int t = 0; t < tn; t++) {
-            const size_t r = (size_t)(t0 + t);
-            xs[t * 64 + lane] = live ? ld_f32((const T*)a.xbc + r * a.xbc_stride + (size_t)head * P + p) : 0.f;
-            if (MODE != 1) zs[t * 64 + lane] = live ? ld_f32((const T*)a.z + r * a.z_stride + (size_t)head * P + p) : 0.f;
+#pragma unroll
+        for (int i = 0; i < TC / 4; i++) {               // row q + 4 i of the round, the lane's channel
+            const size_t r = (size_t)(t0 + min(q + 4 * i, tn - 1));
+            rx[i] = *((const T*)a.xbc + r * a.xbc_stride + (size_t)head * P + pl);
+            if (MODE != 1) rz[i] = *((const T*)a.z + r * a.z_stride + (size_t)head * P + pl);
         }
-        if (lane < tn) {
-            const float d = softplus_f(ld_f32((const T*)a.dt + (size_t)(t0 + lane) * a.dt_stride + head) + bias);
-            dts[lane] = d;
-            dec[lane] = expf(-rate * d);
+        const float draw = ld_f32((const T*)a.dt + (size_t)(t0 + min(tid, tn - 1)) * a.dt_stride + head);
+        __syncthreads();                                 // the round before has been read by every wave
+#pragma unroll
+        for (int j = 0; j < J; j++) {
+            const int c = tid + 256 * j;
+            if (c < packs) {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) { Bs[c * VEC + e] = ld_f32(&rb[j].v[e]); Cs[c * VEC + e] = ld_f32(&rc[j].v[e]); }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TC / 4; i++) {
+            xs[(q + 4 * i) * 64 + lane] = live ? ld_f32(&rx[i]) : 0.f;
+            if (MODE != 1) zs[(q + 4 * i) * 64 + lane] = live ? ld_f32(&rz[i]) : 0.f;
+        }
+        if (tid < tn) {
+            const float d = softplus_f(draw + bias);
+            dts[tid] = d;
+            dec[tid] = expf(-rate * d);
         }
         __syncthreads();
         for (int t = 0; t < tn; t++) {
             const float x = xs[t * 64 + lane];
             const float d = dec[t], dx = dts[t] * x;
-            const float* Bt = Bs + t * N; const float* Ct = Cs + t * N;
+            const float* Bt = Bs + t * N + n0; const float* Ct = Cs + t * N + n0;
             float acc = 0.f;
 #pragma unroll
-            for (int n = 0; n < NR; n++) {
-                if (FULL || n < N) {
+            for (int n = 0; n < NQ; n++) {
+                if (FULL || n0 + n < N) {
                     S[n] = __builtin_fmaf(d, S[n], dx * Bt[n]);
                     if (MODE != 1) acc = __builtin_fmaf(S[n], Ct[n], acc);
                 }
             }
             if (MODE == 1) total *= d;
-            else if (live) {
-                const float zz = zs[t * 64 + lane];
-                a.y[(size_t)(t0 + t) * inner + (size_t)head * P + p] = __builtin_fmaf(skip, x, acc) * (zz / (1.f + expf(-zz)));
+            else parts[(q * TC + t) * 64 + lane] = acc;
+        }
+        if (MODE != 1) {
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < TC / 4; i++) {           // row q + 4 i of the round: the four waves' parts in wave order
+                const int t = q + 4 * i;
+                if (t < tn && live) {
+                    const float acc = ((parts[t * 64 + lane] + parts[(TC + t) * 64 + lane]) + parts[(2 * TC + t) * 64 + lane]) +
+                                      parts[(3 * TC + t) * 64 + lane];
+                    const float zz = zs[t * 64 + lane];
+                    a.y[(size_t)(t0 + t) * inner + (size_t)head * P + p] = __builtin_fmaf(skip, xs[t * 64 + lane], acc) * (zz / (1.f + expf(-zz)));
+                }
             }
         }
     }
@@ -175,12 +275,12 @@ ssd_scan_k(SsdArgs a) {
         float* to = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
         if (live) {
 #pragma unroll
-            for (int n = 0; n < NR; n++) if (FULL || n < N) to[(size_t)n * P] = S[n];
+            for (int n = 0; n < NQ; n++) if (FULL || n0 + n < N) to[(size_t)(n0 + n) * P] = S[n];
         }
-        if (pc == 0 && lane == 0) a.decay[((size_t)seq * a.max_chunks + piece) * a.heads + head] = total;
+        if (pc == 0 && tid == 0) a.decay[((size_t)seq * a.max_chunks + piece) * a.heads + head] = total;
     } else if (last_piece && live) {
 #pragma unroll
-        for (int n = 0; n < NR; n++) if (FULL || n < N) slot_state[(size_t)n * P] = S[n];
+        for (int n = 0; n < NQ; n++) if (FULL || n0 + n < N) slot_state[(size_t)(n0 + n) * P] = S[n];
     }
 }
 
@@ -205,7 +305,13 @@ ssd_carry_k(SsdArgs a) {
 
 template <typename T, int MODE>
 static int launch_scan(const SsdArgs& a, dim3 grid, size_t lds, hipStream_t s) {
-#define TP_SSD(NR) do { if (a.N == NR) ssd_scan_k<T, NR, MODE, true><<<grid, 64, lds, s>>>(a); else ssd_scan_k<T, NR, MODE, false><<<grid, 64, lds, s>>>(a); } while (0)
+    constexpr int V = sizeof(T) == 2 ? 8 : 4;             // 16 bytes of B or C a load, where rows and sizes allow
+    const bool packs = a.N % V == 0 && a.xbc_stride % V == 0 && ((size_t)a.heads * a.P) % V == 0 && (uintptr_t)a.xbc % 16 == 0;
+#define TP_SSD(NR) do { \
+        if (a.N == NR && packs) ssd_scan_k<T, NR, MODE, true, V><<<grid, 256, lds, s>>>(a); \
+        else if (a.N == NR) ssd_scan_k<T, NR, MODE, true, 1><<<grid, 256, lds, s>>>(a); \
+        else if (packs) ssd_scan_k<T, NR, MODE, false, V><<<grid, 256, lds, s>>>(a); \
+        else ssd_scan_k<T, NR, MODE, false, 1><<<grid, 256, lds, s>>>(a); } while (0)
     if (a.N <= 16) TP_SSD(16);
     else if (a.N <= 32) TP_SSD(32);
     else if (a.N <= 64) TP_SSD(64);
@@ -237,7 +343,7 @@ extern "C" int tp_ssd_scan(const void* xbc, long xbc_stride, const void* z, long
     a.xbc = xbc; a.xbc_stride = xbc_stride; a.z = z; a.z_stride = z_stride; a.dt = dt; a.dt_stride = dt_stride;
     a.dt_bias = dt_bias; a.a_log = a_log; a.skip = skip; a.state = state; a.slot_ids = slot_ids; a.cu_rows = cu_rows; a.y = y;
     a.heads = heads; a.groups = groups; a.N = N; a.P = P;
-    const size_t lds = (size_t)(2 * 16 * N + 32 + 2 * 16 * 64) * sizeof(float);
+    const size_t lds = (size_t)(2 * 16 * N + 32 + 6 * 16 * 64) * sizeof(float);
     const int pcs = (P + 63) / 64;
     const long need = tp_ssd_scan_workspace_bytes(n_seq, max_count, heads, N, P, chunk);
     if (need == 0) {
