@@ -59,7 +59,12 @@ class StateSpaceMixer(Mixer):
     def bind(self, tensors, rt):
         self.rt = rt
         n = self.names
-        self.w_in = rt.matrix(tensors[n["in"]])
+        import torch
+        w_in = tensors[n["in"]]
+        spare = -w_in.shape[0] % 8           # zero rows, so that a row of the product is whole 16-byte pieces: the
+        if spare:                            # convolution then reads its columns of it eight elements a load
+            w_in = torch.cat([w_in, w_in.new_zeros((spare, w_in.shape[1]))], dim=0)
+        self.w_in = rt.matrix(w_in.contiguous())
         self.conv_t = tensors[n["conv"]].float().t().contiguous()          # [taps, channels]
         self.conv_b = tensors[n["conv_b"]].float().contiguous()
         self.dt_bias = tensors[n["dt_bias"]].float().contiguous()
@@ -75,7 +80,7 @@ class StateSpaceMixer(Mixer):
         conv_state = self.state(ctx, "conv") if self.taps > 1 else None
         xbc = ops.conv_act(u[:, inner:inner + ch], self.conv_t, self.conv_b, conv_state, ctx.slot_ids, ctx.cu_rows, ctx.row_seq,
                            activation="silu", one_row_each=ctx.mode == "decode")
-        y = ops.ssd_scan(xbc, u[:, :inner], u[:, inner + ch:], self.dt_bias, self.a_log, self.skip, self.state(ctx, "ssm"),
+        y = ops.ssd_scan(xbc, u[:, :inner], u[:, inner + ch:inner + ch + self.num_heads], self.dt_bias, self.a_log, self.skip, self.state(ctx, "ssm"),
                          ctx.slot_ids, ctx.cu_rows, ctx.max_count, self.num_heads, self.groups, self.state_size, self.head_dim)
         y = ops.rms_norm(y, self.norm_gain, self.norm_eps, ctx.dtype, groups=self.norm_groups)
         return ops.linear(y, self.w_o, ctx.dtype, defer=True)
