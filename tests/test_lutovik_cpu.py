@@ -158,3 +158,28 @@ def test_greedy_generation_through_the_loop(m):
     cache = model.new_cache(max_tokens=64 * 2, page_size=64)             # room for two sequences at a time: slots are used again
     assert generate(model, cache, prompts, max_tokens=6, stop_ids=()) == want
     assert cache.live_slots() == [] and cache.tokens_held() == 0
+
+
+@pytest.mark.parametrize("case", range(6))
+def test_random_configuration(case, tmp_path):
+    """A configuration drawn at random: a prompt whole, then in two portions and single tokens."""
+    import random
+
+    from trapetum_amd.weights import write_model_folder
+
+    from .lutovik_random import draw
+    rng = random.Random(500 + case)
+    cfg = draw(rng)
+    folder = str(tmp_path)
+    write_model_folder(LutovikConfig.from_dict(cfg), folder, seed=case, sigma=0.1, sigma_norm=0.2)
+    model, c = load_cpu_model(folder)
+    pcfg, pw = plain.read_folder(folder)
+    assert pcfg == cfg
+    toks = random_tokens(37, c.vocab_size, case)
+    ref = plain.forward(pcfg, pw, toks)
+    cache = model.new_cache(max_tokens=128, page_size=16)
+    s = cache.acquire()
+    got = [model.step(cache, [s], toks[:20], counts=[20], want=list(range(20))),
+           model.step(cache, [s], toks[20:31], counts=[11], want=list(range(11)))]
+    got += [model.step(cache, [s], [t]) for t in toks[31:]]
+    mc.rows_close(torch.cat(got), ref, 5e-5, cfg)
