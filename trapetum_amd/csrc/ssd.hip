@@ -157,28 +157,27 @@ struct SsdArgs {
 
 __device__ __forceinline__ float softplus_f(float v) { return log1pf(expf(-fabsf(v))) + fmaxf(v, 0.f); }
 
-// A block of four waves owns 64 value channels of one head of one sequence (or of one piece of it): wave q keeps a
-// quarter of the state's rows, lane p column p of them, NR / 4 elements in registers, so that several blocks fit a
-// SIMD and one's waits are another's work.  The rows' B and C vectors, step sizes, decays, inputs and gates are staged
-// in LDS TC rows at a time (every load of a round is asked for at once); a row then costs a lane 3 N / 4 vector
-// instructions, and the four waves' parts of y meet in LDS once a round.  FULL: N == NR, no bounds in the inner loop.
-// VEC: elements of B and C a load takes.
+// A block of four waves owns R units of one group of heads, a unit being 64 value channels of one head: wave q keeps a
+// quarter of the state's rows, lane p column p of them for each of the R units, R NR / 4 elements in registers, so that
+// several blocks fit a SIMD and one's waits are another's work.  The rows' B and C vectors (one pair for the whole
+// group, read from LDS once for all R units), step sizes, decays, inputs and gates are staged in LDS TC rows at a time
+// (every load of a round is asked for at once); a row then costs a lane 3 R N / 4 vector instructions, and the four
+// waves' parts of y meet in LDS once a round.  Rows of B and C stand NR apart in LDS, zero beyond N, so the inner loop
+// has no bounds.  VEC: elements of B and C a load takes.
 // MODE 0: the whole scan from the slot's state, which it leaves updated.
 // MODE 1: a piece (not the last) from a zero state: writes the state it ends with and its total decay, no outputs.
 // MODE 2: a piece from the state `carry` holds for its start: writes outputs; the last piece leaves the slot's state.
-template <typename T, int NR, int MODE, bool FULL, int VEC>
+template <typename T, int NR, int MODE, int VEC, int R>
 __global__ void __launch_bounds__(256)
 ssd_scan_k(SsdArgs a) {
-    constexpr int TC = 16, NQ = NR / 4;
+    constexpr int TC = 16 / R, NQ = NR / 4, PAIRS = TC * R;        // PAIRS = 16 (row, unit) pairs a round
     constexpr int J = (TC * NR / VEC + 255) / 256;       // packs of B (and of C) a thread stages a round
     using Pk = Pack<T, VEC>;
-    extern __shared__ float lds[];                       // B [TC][N], C [TC][N], dt [TC], decay [TC], x [TC][64], z [TC][64], parts [4][TC][64]
-    const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
-    const int pieces_z = MODE == 0 ? 1 : a.max_chunks;
-    const int piece = MODE == 0 ? 0 : blockIdx.z % pieces_z, pc = MODE == 0 ? blockIdx.z : blockIdx.z / pieces_z;
-    const int p = pc * 64 + lane;
-    const bool live = p < a.P;
-    const int N = FULL ? NR : a.N, P = a.P, g = head / (a.heads / a.groups);
+    extern __shared__ float lds[];                       // B [TC][NR], C [TC][NR], dt [PAIRS], decay [PAIRS], x [PAIRS][64], z [PAIRS][64], parts [4][PAIRS][64]
+    const int seq = blockIdx.x, tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
+    const int N = a.N, P = a.P, hpg = a.heads / a.groups, pcs = (P + 63) / 64, units = hpg * pcs, bpg = (units + R - 1) / R;
+    const int g = blockIdx.y / bpg, u0 = (blockIdx.y - g * bpg) * R;
+    const int piece = MODE == 0 ? 0 : blockIdx.z;
     const int first = a.cu_rows[seq], count = a.cu_rows[seq + 1] - first;
     int r0 = first, r1 = first + count;
     if (MODE != 0) {
@@ -188,26 +187,35 @@ ssd_scan_k(SsdArgs a) {
     }
     const bool last_piece = MODE == 0 || r1 == first + count;
     if (MODE == 1 && last_piece) return;                 // nobody starts from the state the last piece ends with
-    float* Bs = lds; float* Cs = lds + TC * N; float* dts = Cs + TC * N; float* dec = dts + TC;
-    float* xs = dec + TC; float* zs = xs + TC * 64; float* parts = zs + TC * 64;
-    const float rate = expf(a.a_log[head]), bias = a.dt_bias[head], skip = a.skip[head];
+    float* Bs = lds; float* Cs = lds + TC * NR; float* dts = Cs + TC * NR; float* dec = dts + PAIRS;
+    float* xs = dec + PAIRS; float* zs = xs + PAIRS * 64; float* parts = zs + PAIRS * 64;
+    // unit r of the block: its head, the lane's channel, whether the lane has one
+    auto head_of = [&](int r) { return g * hpg + min(u0 + r, units - 1) / pcs; };
+    auto chan_of = [&](int r) { return (min(u0 + r, units - 1) % pcs) * 64 + lane; };
+    auto live_of = [&](int r) { return u0 + r < units && chan_of(r) < P; };
     const int n0 = q * NQ;                               // the wave's rows of the state
-    float S[NQ];
-    float* slot_state = a.state + (((size_t)a.slot_ids[seq] * a.heads + head) * N) * P + p;
-    const float* from = slot_state;
-    if (MODE == 2) from = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
+    float S[R][NQ], total[R];
 #pragma unroll
-    for (int n = 0; n < NQ; n++) S[n] = (MODE != 1 && live && (FULL || n0 + n < N)) ? from[(size_t)(n0 + n) * P] : 0.f;
-    float total = 1.f;
+    for (int r = 0; r < R; r++) {
+        const int head = head_of(r), p = chan_of(r);
+        const float* from = a.state + (((size_t)a.slot_ids[seq] * a.heads + head) * N) * P + p;
+        if (MODE == 2) from = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
+        const bool live = live_of(r);
+#pragma unroll
+        for (int n = 0; n < NQ; n++) S[r][n] = (MODE != 1 && live && n0 + n < N) ? from[(size_t)(n0 + n) * P] : 0.f;
+        total[r] = 1.f;
+    }
+    if (N < NR) {                                        // the columns beyond N stay zero
+        for (int i = tid; i < 2 * TC * NR; i += 256) lds[i] = 0.f;
+    }
     const size_t inner = (size_t)a.heads * P;
-    const int pl = live ? p : 0;
     for (int t0 = r0; t0 < r1; t0 += TC) {
         const int tn = min(TC, r1 - t0);
         // every load of the round is asked for before the first is used (loads past the round's end read its last row,
         // from an address that exists, and are dropped): a round waits for memory once
         const int per_row = N / VEC, packs = tn * per_row;
         Pk rb[J], rc[J];
-        T rx[TC / 4], rz[TC / 4];
+        T rx[4], rz[4];
 #pragma unroll
         for (int j = 0; j < J; j++) {
             const int c = min(tid + 256 * j, packs - 1), t = c / per_row, k = c - t * per_row;
@@ -216,71 +224,94 @@ ssd_scan_k(SsdArgs a) {
             rc[j] = *reinterpret_cast<const Pk*>(row + (size_t)a.groups * N);
         }
 #pragma unroll
-        for (int i = 0; i < TC / 4; i++) {               // row q + 4 i of the round, the lane's channel
-            const size_t r = (size_t)(t0 + min(q + 4 * i, tn - 1));
-            rx[i] = *((const T*)a.xbc + r * a.xbc_stride + (size_t)head * P + pl);
-            if (MODE != 1) rz[i] = *((const T*)a.z + r * a.z_stride + (size_t)head * P + pl);
+        for (int i = 0; i < 4; i++) {                    // pair q + 4 i of the round: row (q + 4 i) / R, unit (q + 4 i) % R
+            const int pr = q + 4 * i, t = pr / R, r = pr % R;
+            const size_t row = (size_t)(t0 + min(t, tn - 1));
+            const int p = live_of(r) ? chan_of(r) : 0;
+            rx[i] = *((const T*)a.xbc + row * a.xbc_stride + (size_t)head_of(r) * P + p);
+            if (MODE != 1) rz[i] = *((const T*)a.z + row * a.z_stride + (size_t)head_of(r) * P + p);
         }
-        const float draw = ld_f32((const T*)a.dt + (size_t)(t0 + min(tid, tn - 1)) * a.dt_stride + head);
+        const int mt = min(tid, PAIRS - 1) / R, mr = min(tid, PAIRS - 1) % R;
+        const float draw = ld_f32((const T*)a.dt + (size_t)(t0 + min(mt, tn - 1)) * a.dt_stride + head_of(mr));
         __syncthreads();                                 // the round before has been read by every wave
 #pragma unroll
         for (int j = 0; j < J; j++) {
             const int c = tid + 256 * j;
             if (c < packs) {
+                const int t = c / per_row, k = c - t * per_row;
 #pragma unroll
-                for (int e = 0; e < VEC; e++) { Bs[c * VEC + e] = ld_f32(&rb[j].v[e]); Cs[c * VEC + e] = ld_f32(&rc[j].v[e]); }
+                for (int e = 0; e < VEC; e++) { Bs[t * NR + k * VEC + e] = ld_f32(&rb[j].v[e]); Cs[t * NR + k * VEC + e] = ld_f32(&rc[j].v[e]); }
             }
         }
 #pragma unroll
-        for (int i = 0; i < TC / 4; i++) {
-            xs[(q + 4 * i) * 64 + lane] = live ? ld_f32(&rx[i]) : 0.f;
-            if (MODE != 1) zs[(q + 4 * i) * 64 + lane] = live ? ld_f32(&rz[i]) : 0.f;
+        for (int i = 0; i < 4; i++) {
+            const int pr = q + 4 * i, r = pr % R;
+            xs[pr * 64 + lane] = live_of(r) ? ld_f32(&rx[i]) : 0.f;
+            if (MODE != 1) zs[pr * 64 + lane] = live_of(r) ? ld_f32(&rz[i]) : 0.f;
         }
-        if (tid < tn) {
-            const float d = softplus_f(draw + bias);
+        if (tid < PAIRS) {
+            const int head = head_of(mr);
+            const float d = softplus_f(draw + a.dt_bias[head]);
             dts[tid] = d;
-            dec[tid] = expf(-rate * d);
+            dec[tid] = expf(-expf(a.a_log[head]) * d);
         }
         __syncthreads();
         for (int t = 0; t < tn; t++) {
-            const float x = xs[t * 64 + lane];
-            const float d = dec[t], dx = dts[t] * x;
-            const float* Bt = Bs + t * N + n0; const float* Ct = Cs + t * N + n0;
-            float acc = 0.f;
+            float d[R], dx[R], acc[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                d[r] = dec[t * R + r];
+                dx[r] = dts[t * R + r] * xs[(t * R + r) * 64 + lane];
+                acc[r] = 0.f;
+            }
+            const float* Bt = Bs + t * NR + n0; const float* Ct = Cs + t * NR + n0;
 #pragma unroll
             for (int n = 0; n < NQ; n++) {
-                if (FULL || n0 + n < N) {
-                    S[n] = __builtin_fmaf(d, S[n], dx * Bt[n]);
-                    if (MODE != 1) acc = __builtin_fmaf(S[n], Ct[n], acc);
+                const float bn = Bt[n], cn = Ct[n];
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    S[r][n] = __builtin_fmaf(d[r], S[r][n], dx[r] * bn);
+                    if (MODE != 1) acc[r] = __builtin_fmaf(S[r][n], cn, acc[r]);
                 }
             }
-            if (MODE == 1) total *= d;
-            else parts[(q * TC + t) * 64 + lane] = acc;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if (MODE == 1) total[r] *= d[r];
+                else parts[(q * PAIRS + t * R + r) * 64 + lane] = acc[r];
+            }
         }
         if (MODE != 1) {
             __syncthreads();
 #pragma unroll
-            for (int i = 0; i < TC / 4; i++) {           // row q + 4 i of the round: the four waves' parts in wave order
-                const int t = q + 4 * i;
-                if (t < tn && live) {
-                    const float acc = ((parts[t * 64 + lane] + parts[(TC + t) * 64 + lane]) + parts[(2 * TC + t) * 64 + lane]) +
-                                      parts[(3 * TC + t) * 64 + lane];
-                    const float zz = zs[t * 64 + lane];
-                    a.y[(size_t)(t0 + t) * inner + (size_t)head * P + p] = __builtin_fmaf(skip, xs[t * 64 + lane], acc) * (zz / (1.f + expf(-zz)));
+            for (int i = 0; i < 4; i++) {                // pair q + 4 i of the round: the four waves' parts in wave order
+                const int pr = q + 4 * i, t = pr / R, r = pr % R;
+                if (t < tn && live_of(r)) {
+                    const float acc = ((parts[pr * 64 + lane] + parts[(PAIRS + pr) * 64 + lane]) + parts[(2 * PAIRS + pr) * 64 + lane]) +
+                                      parts[(3 * PAIRS + pr) * 64 + lane];
+                    const float zz = zs[pr * 64 + lane];
+                    const int head = head_of(r);
+                    a.y[(size_t)(t0 + t) * inner + (size_t)head * P + chan_of(r)] =
+                        __builtin_fmaf(a.skip[head], xs[pr * 64 + lane], acc) * (zz / (1.f + expf(-zz)));
                 }
             }
         }
     }
-    if (MODE == 1) {
-        float* to = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
-        if (live) {
 #pragma unroll
-            for (int n = 0; n < NQ; n++) if (FULL || n0 + n < N) to[(size_t)(n0 + n) * P] = S[n];
+    for (int r = 0; r < R; r++) {
+        if (u0 + r >= units) continue;
+        const int head = head_of(r), p = chan_of(r);
+        if (MODE == 1) {
+            float* to = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
+            if (p < P) {
+#pragma unroll
+                for (int n = 0; n < NQ; n++) if (n0 + n < N) to[(size_t)(n0 + n) * P] = S[r][n];
+            }
+            if (tid == 0 && (u0 + r) % pcs == 0) a.decay[((size_t)seq * a.max_chunks + piece) * a.heads + head] = total[r];
+        } else if (last_piece && p < P) {
+            float* slot_state = a.state + (((size_t)a.slot_ids[seq] * a.heads + head) * N) * P + p;
+#pragma unroll
+            for (int n = 0; n < NQ; n++) if (n0 + n < N) slot_state[(size_t)(n0 + n) * P] = S[r][n];
         }
-        if (pc == 0 && tid == 0) a.decay[((size_t)seq * a.max_chunks + piece) * a.heads + head] = total;
-    } else if (last_piece && live) {
-#pragma unroll
-        for (int n = 0; n < NQ; n++) if (FULL || n0 + n < N) slot_state[(size_t)(n0 + n) * P] = S[n];
     }
 }
 
@@ -303,20 +334,30 @@ ssd_carry_k(SsdArgs a) {
     }
 }
 
+// Units of 64 channels a block takes.  Two (where a group of heads has two), which halves the reads of B and C from LDS,
+// measured the same as one (217 against 219 us for 2,048 rows of 36 heads x 64 channels with a state of 128) at fewer waves
+// a SIMD: the kernel keeps the parameter, one unit is what is compiled.
+static int scan_units(const SsdArgs&) { return 1; }
+static int scan_nr(int N) { return N <= 16 ? 16 : N <= 32 ? 32 : N <= 64 ? 64 : N <= 128 ? 128 : 256; }
+static size_t scan_lds(int N) { return (size_t)(2 * 16 * scan_nr(N) + 32 + 6 * 16 * 64) * sizeof(float); }     // 16 rows x 1 unit, or 8 x 2
+
 template <typename T, int MODE>
-static int launch_scan(const SsdArgs& a, dim3 grid, size_t lds, hipStream_t s) {
+static int launch_scan(const SsdArgs& a, int n_seq, int pieces, hipStream_t s) {
     constexpr int V = sizeof(T) == 2 ? 8 : 4;             // 16 bytes of B or C a load, where rows and sizes allow
     const bool packs = a.N % V == 0 && a.xbc_stride % V == 0 && ((size_t)a.heads * a.P) % V == 0 && (uintptr_t)a.xbc % 16 == 0;
+    const int R = scan_units(a), units = (a.heads / a.groups) * ((a.P + 63) / 64);
+    dim3 grid(n_seq, a.groups * ((units + R - 1) / R), pieces);
+    const size_t lds = scan_lds(a.N);
 #define TP_SSD(NR) do { \
-        if (a.N == NR && packs) ssd_scan_k<T, NR, MODE, true, V><<<grid, 256, lds, s>>>(a); \
-        else if (a.N == NR) ssd_scan_k<T, NR, MODE, true, 1><<<grid, 256, lds, s>>>(a); \
-        else if (packs) ssd_scan_k<T, NR, MODE, false, V><<<grid, 256, lds, s>>>(a); \
-        else ssd_scan_k<T, NR, MODE, false, 1><<<grid, 256, lds, s>>>(a); } while (0)
-    if (a.N <= 16) TP_SSD(16);
-    else if (a.N <= 32) TP_SSD(32);
-    else if (a.N <= 64) TP_SSD(64);
-    else if (a.N <= 128) TP_SSD(128);
-    else TP_SSD(256);
+        if (packs) ssd_scan_k<T, NR, MODE, V, 1><<<grid, 256, lds, s>>>(a); \
+        else ssd_scan_k<T, NR, MODE, 1, 1><<<grid, 256, lds, s>>>(a); } while (0)
+    switch (scan_nr(a.N)) {
+        case 16: TP_SSD(16); break;
+        case 32: TP_SSD(32); break;
+        case 64: TP_SSD(64); break;
+        case 128: TP_SSD(128); break;
+        default: TP_SSD(256);
+    }
 #undef TP_SSD
     return tp_check_launch("ssd_scan");
 }
@@ -335,7 +376,6 @@ extern "C" int tp_ssd_scan(const void* xbc, long xbc_stride, const void* z, long
     TP_REQUIRE(n_seq > 0 && max_count > 0 && heads > 0 && groups > 0 && N > 0 && P > 0, "ssd_scan: empty shape sequences=%d heads=%d groups=%d N=%d P=%d", n_seq, heads, groups, N, P);
     TP_REQUIRE(heads % groups == 0, "ssd_scan: %d heads are no multiple of %d groups", heads, groups);
     TP_REQUIRE(N <= 256, "ssd_scan: a state of %d rows per head exceeds 256", N);
-    TP_REQUIRE(heads <= 65535 && (P + 63) / 64 <= 65535, "ssd_scan: too many heads or channels for one launch");
     TP_REQUIRE(xbc && z && dt && dt_bias && a_log && skip && state && slot_ids && cu_rows && y, "ssd_scan: a null operand");
     TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F32, "ssd_scan: unknown dtype %d", dtype);
     hipStream_t s = (hipStream_t)stream;
@@ -343,23 +383,19 @@ extern "C" int tp_ssd_scan(const void* xbc, long xbc_stride, const void* z, long
     a.xbc = xbc; a.xbc_stride = xbc_stride; a.z = z; a.z_stride = z_stride; a.dt = dt; a.dt_stride = dt_stride;
     a.dt_bias = dt_bias; a.a_log = a_log; a.skip = skip; a.state = state; a.slot_ids = slot_ids; a.cu_rows = cu_rows; a.y = y;
     a.heads = heads; a.groups = groups; a.N = N; a.P = P;
-    const size_t lds = (size_t)(2 * 16 * N + 32 + 6 * 16 * 64) * sizeof(float);
-    const int pcs = (P + 63) / 64;
+    TP_REQUIRE((long)a.groups * (a.heads / a.groups) * ((P + 63) / 64) <= 65535, "ssd_scan: too many heads or channels for one launch");
     const long need = tp_ssd_scan_workspace_bytes(n_seq, max_count, heads, N, P, chunk);
-    if (need == 0) {
-        dim3 grid(n_seq, heads, pcs);
-        return dtype == TP_BF16 ? launch_scan<bf16_t, 0>(a, grid, lds, s) : launch_scan<float, 0>(a, grid, lds, s);
-    }
+    if (need == 0)
+        return dtype == TP_BF16 ? launch_scan<bf16_t, 0>(a, n_seq, 1, s) : launch_scan<float, 0>(a, n_seq, 1, s);
     TP_REQUIRE(workspace && workspace_bytes >= need, "ssd_scan: a workspace of %ld bytes is too small (%ld)", workspace_bytes, need);
     a.chunk = chunk; a.max_chunks = (max_count + chunk - 1) / chunk;
-    TP_REQUIRE((long)pcs * a.max_chunks <= 65535, "ssd_scan: %d pieces exceed one launch", a.max_chunks);
+    TP_REQUIRE(a.max_chunks <= 65535, "ssd_scan: %d pieces exceed one launch", a.max_chunks);
     a.carry = (float*)workspace;
     a.decay = a.carry + (size_t)n_seq * a.max_chunks * heads * N * P;
-    dim3 grid(n_seq, heads, pcs * a.max_chunks);
-    if (int rc = dtype == TP_BF16 ? launch_scan<bf16_t, 1>(a, grid, lds, s) : launch_scan<float, 1>(a, grid, lds, s)) return rc;
+    if (int rc = dtype == TP_BF16 ? launch_scan<bf16_t, 1>(a, n_seq, a.max_chunks, s) : launch_scan<float, 1>(a, n_seq, a.max_chunks, s)) return rc;
     ssd_carry_k<<<dim3(n_seq, heads, tp_cdiv((long)N * P, 256)), 256, 0, s>>>(a);
     if (int rc = tp_check_launch("ssd_scan (carry)")) return rc;
-    return dtype == TP_BF16 ? launch_scan<bf16_t, 2>(a, grid, lds, s) : launch_scan<float, 2>(a, grid, lds, s);
+    return dtype == TP_BF16 ? launch_scan<bf16_t, 2>(a, n_seq, a.max_chunks, s) : launch_scan<float, 2>(a, n_seq, a.max_chunks, s);
 }
 
 // ---- 0.5 (a / rms(a) * wa + b / rms(b) * wb), one block a row ------------------------------------------------------------
