@@ -207,7 +207,7 @@ def _attend(qrow, keys, vals, scale, softcap):
 
 
 def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype, row_seq=None, row_pos=None,
-                      cached=None, shape=0):
+                      cached=None, shape=0, wide_weights=False):
     """k, v: the step's own rows.  cached None: every sequence starts at position 0.  Else cached = (new_len, table,
     k_pool, v_pool, rows_cap): sequence i's first row stands at new_len[i] - its count, and the positions before it are
     read from the cache as it is."""

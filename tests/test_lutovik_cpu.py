@@ -89,7 +89,7 @@ def test_config_errors():
         LutovikConfig.from_dict(d)
 
 
-@pytest.mark.parametrize("base,dims,scaling", [(500.0, 8, (8.0, 1.0, 3.0, 64)), (10000.0, 32, (4.0, 1.0, 4.0, 256)),
+@pytest.mark.parametrize("base,dims,scaling", [(500.0, 8, (8.0, 1.0, 3.0, 64)), (10000.0, 32, (6.0, 1.0, 5.0, 256)),
                                                (3000.0, 12, (2.5, 2.0, 9.0, 100)), (77.0, 24, None)])
 def test_scaled_frequencies(base, dims, scaling):
     sc = None if scaling is None else dict(zip(("factor", "low", "high", "original"), scaling))

@@ -105,7 +105,7 @@ def attention_part(rt, H, G, dim, vdim, rot, pairing, scaling=None, gate=False, 
         edit(T)
     part, W = bound(rt, "mixer", ("attention", dict(
         hidden_size=WIDTH, num_heads=H, num_kv_heads=G, head_dim=dim, value_dim=vdim, query_scale=scale, position=position,
-        output_gate=gate, own_kv=own, tensors=("q", "k", "v", "o", "g"))), T)
+        output_gate=gate, own_kv=own, precise_weights=True, tensors=("q", "k", "v", "o", "g"))), T)
     sizes = {"heads": H, "kv_heads": G, "dim": dim, "vdim": vdim, "scale": scale, "rot": {"base": 300.0, "dims": rot}}
     if sc is not None:
         sizes["rot"]["scaling"] = sc
@@ -114,7 +114,7 @@ def attention_part(rt, H, G, dim, vdim, rot, pairing, scaling=None, gate=False, 
 
 @pytest.mark.parametrize("H,G,dim,vdim,rot,pairing,scaling,gate", [
     (4, 2, 16, 24, 8, "neighbours", (8.0, 1.0, 3.0, 64), False), (2, 1, 32, 16, 32, "halves", None, True),
-    (6, 3, 64, 64, 16, "neighbours", (4.0, 1.0, 4.0, 128), False), (4, 4, 48, 80, 48, "halves", None, True),
+    (10, 5, 64, 64, 24, "neighbours", (3.0, 2.0, 8.0, 100), False), (4, 4, 48, 80, 48, "halves", None, True),
     (1, 1, 12, 12, 0, "halves", None, True), (3, 1, 20, 36, 6, "neighbours", None, True), (8, 2, 128, 64, 64, "neighbours", None, False)])
 def test_attention_part(rt, H, G, dim, vdim, rot, pairing, scaling, gate):
     """The mixer alone, and a second one without key and value projections on the first one's cache."""
@@ -177,7 +177,7 @@ def state_space_part(rt, heads, P, N, groups, taps, norm_groups, seed=0, a_log=N
 
 
 @pytest.mark.parametrize("heads,P,N,groups,taps,norm_groups", [(4, 12, 16, 2, 4, 3), (1, 10, 4, 1, 1, 1), (3, 20, 8, 1, 2, 1),
-                                                              (8, 64, 32, 2, 3, 2), (2, 80, 24, 2, 5, 4), (6, 16, 128, 3, 2, 1),
+                                                              (6, 64, 48, 3, 3, 2), (2, 80, 24, 2, 5, 4), (6, 16, 128, 3, 2, 1),
                                                               (2, 130, 40, 1, 3, 2)])
 def test_state_space_part(rt, heads, P, N, groups, taps, norm_groups):
     part, W, sizes = state_space_part(rt, heads, P, N, groups, taps, norm_groups)
@@ -209,7 +209,7 @@ def test_state_space_keeps_its_first_tokens(rt, cut):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("counts,heads,groups,N,P,taps", [([5], 2, 1, 16, 8, 3), ([1, 1, 1], 4, 2, 32, 48, 3), ([70, 1, 200, 33], 8, 2, 32, 48, 4),
+@pytest.mark.parametrize("counts,heads,groups,N,P,taps", [([5], 2, 1, 16, 8, 3), ([1, 1, 1], 4, 2, 32, 40, 3), ([70, 1, 200, 33], 6, 3, 48, 40, 4),
                                                           ([300], 4, 4, 24, 80, 2), ([130, 65], 2, 1, 128, 64, 1), ([700], 1, 1, 200, 16, 2)])
 def test_conv_and_scan_kernels(dt, counts, heads, groups, N, P, taps):
     """The convolution and the scan against their plain torch references, from states that are not zero, in slots that are

@@ -51,7 +51,7 @@ def lutovik_config(which, layers=0):
     D, I, H, KV, hd = g["hidden_size"], g["intermediate_size"], g["num_attention_heads"], g["num_key_value_heads"], g["head_dim"]
     rot = {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
     att = {"heads": H, "kv_heads": KV, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "rot": rot}
-    left = {"heads": H, "kv_heads": KV, "dim": hd // 2, "vdim": hd, "scale": (hd // 2) ** -0.5, "rot": {"base": 50000.0, "dims": hd // 2}}
+    left = {"heads": H, "kv_heads": KV, "dim": hd // 2, "vdim": hd, "scale": (hd // 2) ** -0.5, "rot": {"base": 100000.0, "dims": hd // 2}}
     right = {"heads": D // 64, "vdim": 64, "state": 128, "groups": 4, "conv": 4, "norm_groups": 4}
     moe = {"kind": "moe", "expert": {"ff": I // 2}, "router": {"experts": 8, "top": 2}, "shared": {"ff": I // 4}}
     out = []
@@ -343,7 +343,8 @@ def time_lutovik_kernels(engine, cfg, batch, context, prefill_tokens):
                     name=f"attention_ctx{context}", bytes_each=2.0 * batch * context * 2 * KV * row)
             else:
                 q, k, v = (torch.randn((rows, n * row), device=dev).to(bf) for n in (H, KV, KV))
-                one([lambda: ops.attention_prefill(q, k, v, H, KV, row, ctx.cu_rows, rows, a.query_scale, 0.0, 0, bf)] * 4,
+                one([lambda: ops.attention_prefill(q, k, v, H, KV, row, ctx.cu_rows, rows, a.query_scale, 0.0, 0, bf,
+                                                   wide_weights=a.precise_weights)] * 4,
                     name="attention", flops_each=4.0 * (rows * (rows + 1) / 2.0) * H * row)
             # ---- the parallel layers: the gated attention's extras, the state-space mixer, the average of the two
             if par:
@@ -354,14 +355,14 @@ def time_lutovik_kernels(engine, cfg, batch, context, prefill_tokens):
                 one([lambda: ops.mul_sigmoid(heads_out, gates)] * 16, name="mul_sigmoid", bytes_each=rows * left.num_heads * left.row * 6.0)
                 prod("ssm_in_proj", [(lambda b=b: ops.linear(x, b.mixer.sides[1].w_in, bf)) for b in par], right.w_in)
                 inner, ch, nh, N, P = right.inner, right.conv_channels, right.num_heads, right.state_size, right.head_dim
-                u = (torch.randn((rows, inner + ch + nh), device=dev) * 0.5).to(bf)
+                u = (torch.randn((rows, right.w_in.shape[0]), device=dev) * 0.5).to(bf)     # the in-projection's rows, as the mixer gets them
                 conv_state = cache.entry_state(par_entry, "mixer.right.conv") if right.taps > 1 else None
                 ssm_state = cache.entry_state(par_entry, "mixer.right.ssm")
                 conv = lambda: ops.conv_act(u[:, inner:inner + ch], right.conv_t, right.conv_b, conv_state, ctx.slot_ids, ctx.cu_rows, ctx.row_seq,
                                             activation="silu", one_row_each=decode)
                 one([conv] * 16, name="conv_act", bytes_each=rows * ch * 4.0 + (rows * (right.taps - 1) * ch * 8.0 if decode else 0.0))
                 xbc = conv()
-                scan = lambda: ops.ssd_scan(xbc, u[:, :inner], u[:, inner + ch:], right.dt_bias, right.a_log, right.skip, ssm_state, ctx.slot_ids,
+                scan = lambda: ops.ssd_scan(xbc, u[:, :inner], u[:, inner + ch:inner + ch + nh], right.dt_bias, right.a_log, right.skip, ssm_state, ctx.slot_ids,
                                             ctx.cu_rows, rows if not decode else 1, nh, right.groups, N, P)
                 if decode:
                     one([scan] * 8, name="ssd_scan", bytes_each=batch * nh * N * P * 8.0)

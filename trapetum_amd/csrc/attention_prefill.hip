@@ -69,6 +69,13 @@ constexpr int MERGE_LANE = DT * 16 + 4;       // floats a lane hands over: its p
 constexpr int QL = HD > 128 ? 4 : 0, QR = KS16 - QL;
 constexpr int KD = 2, VD = 2;                 // fragments of K (with the query fragment from LDS) and of V asked for ahead of their product
 constexpr float LOG2E = 1.4426950408889634f;
+#ifndef TP_WIDE_WEIGHTS
+#define TP_WIDE_WEIGHTS 0
+#endif
+// The softmax weights are the second product's bf16 operand.  WIDE: a weight goes in as two bf16 terms, its rounding
+// and the rounding's remainder (16 bits of mantissa together, twice the matrix instructions of the second product),
+// for designs that want their attention weights in 32 bits.
+constexpr bool WIDE = TP_WIDE_WEIGHTS != 0;
 constexpr float LAZY = 8.f;                   // the running maximum moves only when a score exceeds it by this much (log 2 units)
 
 // LDS layout of a tile: sub-tile j holds head elements 64 j .. 64 j + 63 as 32 rows (keys) of 128 bytes, whose
@@ -312,13 +319,15 @@ attn_prefill_k(PrefillArgs a) {
             }
             m_ref = m_new;
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            PFrag pf[2];
+            PFrag pf[2], pl[2];
             float sum = 0.f;
 #pragma unroll
             for (int j = 0; j < 16; j++) {
                 const float p = exp2_fast(sc[j] - m_use);
                 sum += p;
-                pf[j >> 3].v[j & 7] = (__bf16)p;
+                const __bf16 hi = (__bf16)p;
+                pf[j >> 3].v[j & 7] = hi;
+                if constexpr (WIDE) pl[j >> 3].v[j & 7] = (__bf16)(p - (float)hi);
             }
             l_i += sum;
             // fragment i = t * DT + dt of V^T (k step t, head elements dt * 32 ..): the next one is asked for before
@@ -347,6 +356,7 @@ attn_prefill_k(PrefillArgs a) {
             for (int i = 0; i < 2 * DT; i++) {
                 if (i + VD - 1 < 2 * DT) vq[(i + VD - 1) % VD] = v_frag(i + VD - 1);
                 o[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vq[i % VD].v, pf[i / DT].v, o[i % DT], 0, 0, 0);
+                if constexpr (WIDE) o[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vq[i % VD].v, pl[i / DT].v, o[i % DT], 0, 0, 0);
             }
         }
         // the next K tile has landed, and every wave has used the V tile, whose successor may come

@@ -116,8 +116,8 @@ extern "C" int tp_conv_act(const void* x, long x_stride, int in_dtype, const flo
     TP_REQUIRE(in_dtype == out_dtype && (in_dtype == TP_BF16 || in_dtype == TP_F32), "conv_act: rows and output share one dtype, bfloat16 or float32");
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(M, tp_cdiv(C, 256));
-    const int vec = in_dtype == TP_BF16 ? 8 : 4;         // 16 bytes of the rows a thread
-    const bool packs = C % vec == 0 && x_stride % vec == 0 && out_stride % vec == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+    const int vec = in_dtype == TP_BF16 ? 8 : 4;         // 16 bytes of the rows a thread; few rows: a thread a channel, more blocks
+    const bool packs = (long)M * C >= (1L << 18) && C % vec == 0 && x_stride % vec == 0 && out_stride % vec == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0 &&
                        (uintptr_t)wt % 32 == 0 && (!bias || (uintptr_t)bias % 32 == 0) && (!state || (uintptr_t)state % 32 == 0);
     if (packs) {
         dim3 vgrid(M, tp_cdiv(C / vec, 256));
@@ -189,26 +189,49 @@ ssd_scan_k(SsdArgs a) {
     if (MODE == 1 && last_piece) return;                 // nobody starts from the state the last piece ends with
     float* Bs = lds; float* Cs = lds + TC * NR; float* dts = Cs + TC * NR; float* dec = dts + PAIRS;
     float* xs = dec + PAIRS; float* zs = xs + PAIRS * 64; float* parts = zs + PAIRS * 64;
-    // unit r of the block: its head, the lane's channel, whether the lane has one
-    auto head_of = [&](int r) { return g * hpg + min(u0 + r, units - 1) / pcs; };
-    auto chan_of = [&](int r) { return (min(u0 + r, units - 1) % pcs) * 64 + lane; };
-    auto live_of = [&](int r) { return u0 + r < units && chan_of(r) < P; };
+    // unit r of the block: its head, the lane's channel, whether the lane has one (worked out once: the divisions are
+    // as many instructions as a row of the scan)
+    int unit_head[R], unit_chan[R];
+    bool unit_live[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int u = min(u0 + r, units - 1), hl = u / pcs;
+        unit_head[r] = g * hpg + hl;
+        unit_chan[r] = (u - hl * pcs) * 64 + lane;
+        unit_live[r] = u0 + r < units && unit_chan[r] < P;
+    }
+    auto head_of = [&](int r) { int v = unit_head[0]; for (int i = 1; i < R; i++) v = r == i ? unit_head[i] : v; return v; };
+    auto chan_of = [&](int r) { int v = unit_chan[0]; for (int i = 1; i < R; i++) v = r == i ? unit_chan[i] : v; return v; };
+    auto live_of = [&](int r) { bool v = unit_live[0]; for (int i = 1; i < R; i++) v = r == i ? unit_live[i] : v; return v; };
     const int n0 = q * NQ;                               // the wave's rows of the state
     float S[R][NQ], total[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const int head = head_of(r), p = chan_of(r);
+        const bool live = live_of(r);
+        const int head = head_of(r), p = live ? chan_of(r) : 0;
         const float* from = a.state + (((size_t)a.slot_ids[seq] * a.heads + head) * N) * P + p;
         if (MODE == 2) from = a.carry + ((((size_t)seq * a.max_chunks + piece) * a.heads + head) * N) * P + p;
-        const bool live = live_of(r);
+        // all of them asked for at once, from addresses that exist, and masked afterwards: a load behind a condition is
+        // waited for on the spot
+        if (MODE != 1) {
 #pragma unroll
-        for (int n = 0; n < NQ; n++) S[r][n] = (MODE != 1 && live && n0 + n < N) ? from[(size_t)(n0 + n) * P] : 0.f;
+            for (int n = 0; n < NQ; n++) S[r][n] = from[(size_t)min(n0 + n, N - 1) * P];
+        }
+#pragma unroll
+        for (int n = 0; n < NQ; n++) S[r][n] = (MODE != 1 && live && n0 + n < N) ? S[r][n] : 0.f;
         total[r] = 1.f;
     }
     if (N < NR) {                                        // the columns beyond N stay zero
         for (int i = tid; i < 2 * TC * NR; i += 256) lds[i] = 0.f;
     }
     const size_t inner = (size_t)a.heads * P;
+    // what does not change from round to round is fetched once, beside the state: the constants of the head whose step
+    // size this thread prepares, and of the heads whose outputs it stores
+    const int mt = min(tid, PAIRS - 1) / R, mr = min(tid, PAIRS - 1) % R;
+    const float my_bias = a.dt_bias[head_of(mr)], my_rate = expf(a.a_log[head_of(mr)]);
+    float skip[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) skip[r] = a.skip[head_of(r)];
     for (int t0 = r0; t0 < r1; t0 += TC) {
         const int tn = min(TC, r1 - t0);
         // every load of the round is asked for before the first is used (loads past the round's end read its last row,
@@ -231,7 +254,6 @@ ssd_scan_k(SsdArgs a) {
             rx[i] = *((const T*)a.xbc + row * a.xbc_stride + (size_t)head_of(r) * P + p);
             if (MODE != 1) rz[i] = *((const T*)a.z + row * a.z_stride + (size_t)head_of(r) * P + p);
         }
-        const int mt = min(tid, PAIRS - 1) / R, mr = min(tid, PAIRS - 1) % R;
         const float draw = ld_f32((const T*)a.dt + (size_t)(t0 + min(mt, tn - 1)) * a.dt_stride + head_of(mr));
         __syncthreads();                                 // the round before has been read by every wave
 #pragma unroll
@@ -250,10 +272,9 @@ ssd_scan_k(SsdArgs a) {
             if (MODE != 1) zs[pr * 64 + lane] = live_of(r) ? ld_f32(&rz[i]) : 0.f;
         }
         if (tid < PAIRS) {
-            const int head = head_of(mr);
-            const float d = softplus_f(draw + a.dt_bias[head]);
+            const float d = softplus_f(draw + my_bias);
             dts[tid] = d;
-            dec[tid] = expf(-expf(a.a_log[head]) * d);
+            dec[tid] = expf(-my_rate * d);
         }
         __syncthreads();
         for (int t = 0; t < tn; t++) {
@@ -289,9 +310,8 @@ ssd_scan_k(SsdArgs a) {
                     const float acc = ((parts[pr * 64 + lane] + parts[(PAIRS + pr) * 64 + lane]) + parts[(2 * PAIRS + pr) * 64 + lane]) +
                                       parts[(3 * PAIRS + pr) * 64 + lane];
                     const float zz = zs[pr * 64 + lane];
-                    const int head = head_of(r);
-                    a.y[(size_t)(t0 + t) * inner + (size_t)head * P + chan_of(r)] =
-                        __builtin_fmaf(a.skip[head], xs[pr * 64 + lane], acc) * (zz / (1.f + expf(-zz)));
+                    a.y[(size_t)(t0 + t) * inner + (size_t)head_of(r) * P + chan_of(r)] =
+                        __builtin_fmaf(skip[r], xs[pr * 64 + lane], acc) * (zz / (1.f + expf(-zz)));
                 }
             }
         }

@@ -142,9 +142,12 @@ def build_core(force=False):
     return build_library("trapetum_core", CORE_SOURCES, force=force)
 
 
-def attn_name(head_dim):
-    return f"trapetum_attn_hd{head_dim}"
+def attn_name(head_dim, wide=False):
+    return f"trapetum_attn_hd{head_dim}" + ("w" if wide else "")
 
 
-def build_attention(head_dim, force=False):
-    return build_library(attn_name(head_dim), ATTN_SOURCES, [f"-DTP_HD={head_dim}"], force=force)
+def build_attention(head_dim, force=False, wide=False):
+    """wide: the variant whose kernel of many queries carries the softmax weights into the second product as two bf16
+    terms (see attention_prefill.hip)."""
+    defines = [f"-DTP_HD={head_dim}"] + (["-DTP_WIDE_WEIGHTS=1"] if wide else [])
+    return build_library(attn_name(head_dim, wide), ATTN_SOURCES, defines, force=force)

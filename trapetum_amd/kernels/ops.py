@@ -177,15 +177,16 @@ class HipOps:
             raise KernelError(f"{what}: expected rows with contiguous elements, found shape {tuple(t.shape)} strides {t.stride()}")
         return t.stride(0)
 
-    def attn_lib(self, head_dim):
-        if head_dim not in self._attn:
+    def attn_lib(self, head_dim, wide=False):
+        key = (head_dim, bool(wide))
+        if key not in self._attn:
             try:
-                lib = _c.CDLL(_build.build_attention(head_dim))
+                lib = _c.CDLL(_build.build_attention(head_dim, wide=wide))
             except (OSError, _build.BuildError) as e:
                 raise KernelError(f"the attention kernels for head_dim {head_dim} could not be built or loaded: {e}") from None
             _bind(lib, _ATTN_SIGS)
-            self._attn[head_dim] = lib
-        return self._attn[head_dim]
+            self._attn[key] = lib
+        return self._attn[key]
 
     # ---- weights layout ----------------------------------------------------------------------------
     def pack_gate_up(self, w_gate, w_up):
@@ -625,12 +626,14 @@ class HipOps:
             (not decode or H // KV <= self.DECODE_GROUP)
 
     def attention_prefill(self, q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype,
-                          row_seq=None, row_pos=None, cached=None, shape=0):
+                          row_seq=None, row_pos=None, cached=None, shape=0, wide_weights=False):
         """Causal attention of the step's queries over the step's own rows of keys and values and, with
         `cached` = (new_len, table, k_pool, v_pool, rows_cap), over the positions before them, read in place from the
         cache as earlier steps left it (the step's own rows are not looked for there).  Without `cached` every sequence
         starts at position 0; with it row_pos holds absolute positions, sequence s's first row standing at
-        new_len[s] - its count.  shape: the matrix-core kernel's block shape (0: chosen by the size of the step)."""
+        new_len[s] - its count.  shape: the matrix-core kernel's block shape (0: chosen by the size of the step).
+        wide_weights: the matrix-core kernel multiplies the values by softmax weights of 16 bits of mantissa (two bf16
+        terms) instead of 8; the plain kernel's weights are float32 in any case."""
         self._dev(q, k, v, cu_rows)
         m = q.shape[0]
         qs, ks, vs = self._rows(q, "attention q"), self._rows(k, "attention k"), self._rows(v, "attention v")
@@ -649,7 +652,7 @@ class HipOps:
         ptr = lambda t: t.data_ptr() if t is not None else None
         out = torch.empty((m, H * hd), dtype=out_dtype, device=self.device)
         if self._fast_attention(q.dtype, H, KV, hd, decode=False) and (cached is None or (page >= 16 and page & (page - 1) == 0)):
-            lib = self.attn_lib(hd)
+            lib = self.attn_lib(hd, wide=wide_weights)
             self._call(lib, "tp_attn_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs,
                        m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count), ptr(new_len), ptr(table), table_w,
                        ptr(k_pool), ptr(v_pool), page, rows_cap,

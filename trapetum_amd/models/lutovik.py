@@ -21,7 +21,7 @@ def _attention(D, m, pairing, gate=False):
                          "scaling": m.rot.scaling_dict()}) if m.rot.dims else ("none", {})
     return ("attention", {"hidden_size": D, "num_heads": m.heads, "num_kv_heads": m.kv_heads, "head_dim": m.dim,
                           "value_dim": m.vdim, "query_scale": m.scale, "position": position, "output_gate": gate,
-                          "own_kv": m.kv_from is None, "tensors": ("q", "k", "v", "o", "g")})
+                          "own_kv": m.kv_from is None, "precise_weights": True, "tensors": ("q", "k", "v", "o", "g")})
 
 
 def build_spec(c: LutovikConfig) -> ModelSpec:

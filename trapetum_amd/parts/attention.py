@@ -30,11 +30,13 @@ from .base import Mixer
 class Attention(Mixer):
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, query_scale,
                  softcap=None, window=None, position=("none", {}), value_dim=None, output_gate=False, own_kv=True,
+                 precise_weights=False,
                  tensors=("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight", "g_proj.weight")):
         """value_dim: elements of a value head when they differ from a key's head_dim.  output_gate: the heads' outputs
         are multiplied by sigmoid(W_g x) before the output projection.  own_kv False: the layer has no key and value
-        projections; its schedule entry names the run whose cache it reads.  tensors: local names of W_q, W_k, W_v, W_o
-        (and W_g)."""
+        projections; its schedule entry names the run whose cache it reads.  precise_weights: the softmax weights meet
+        the values with 16 bits of mantissa or more in every kernel (the kernel of many queries rounds them to bfloat16
+        otherwise; a decode step's are float32 anyway).  tensors: local names of W_q, W_k, W_v, W_o (and W_g)."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} kv heads")
         self.hidden_size = hidden_size
@@ -51,6 +53,7 @@ class Attention(Mixer):
         self.window = int(window) if window else 0
         self.output_gate = bool(output_gate)
         self.own_kv = bool(own_kv)
+        self.precise_weights = bool(precise_weights)
         self.names = dict(zip(("q", "k", "v", "o", "g"), tuple(tensors) + ("g_proj.weight",) * (5 - len(tensors))))
         self.position = build_part("position", position)
         if self.position.rotary_dim > head_dim:
@@ -157,7 +160,8 @@ class Attention(Mixer):
         out = ops.attention_prefill(q, k, v, H, KV, hd, ctx.cu_rows, ctx.max_count,
                                     self.query_scale, self.softcap, self.window, ctx.dtype,
                                     row_seq=ctx.row_seq, row_pos=ctx.row_pos,
-                                    cached=(ctx.new_len, table, k_pool, v_pool, rows_cap) if extend else None)
+                                    cached=(ctx.new_len, table, k_pool, v_pool, rows_cap) if extend else None,
+                                    wide_weights=self.precise_weights)
         if extend and owns_cache:
             row_seq, row_pos, new_len = ctx.row_seq, ctx.row_pos, ctx.new_len
             ctx.after_readers(lambda: ops.kv_write(k, v, KV, hd, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap))
