@@ -1,10 +1,10 @@
-"""trapetum_amd: Gemma-2 and Golepel generation on one AMD MI355X, assembled from registered parts.
+"""trapetum_amd: Gemma-2, Golepel and Lutovik generation on one AMD MI355X, assembled from registered parts.
 
     from trapetum_amd import load_model
     engine = load_model("path/to/model", dtype="bfloat16")
     ids = engine.generate([[2, 651, 6037]], max_tokens=24)
 """
-from .config import ConfigError, Gemma2Config, GolepelConfig   # noqa: F401
+from .config import ConfigError, Gemma2Config, GolepelConfig, LutovikConfig   # noqa: F401
 from .registry import (architecture, architectures, config_from_folder, register_architecture,   # noqa: F401
                        register_part)
 
