@@ -209,11 +209,13 @@ def test_state_space_keeps_its_first_tokens(rt, cut):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rate", [0.0, 2.5, 4.0])
 @pytest.mark.parametrize("counts,heads,groups,N,P,taps", [([5], 2, 1, 16, 8, 3), ([1, 1, 1], 4, 2, 32, 40, 3), ([70, 1, 200, 33], 6, 3, 48, 40, 4),
                                                           ([300], 4, 4, 24, 80, 2), ([130, 65], 2, 1, 128, 64, 1), ([700], 1, 1, 200, 16, 2)])
-def test_conv_and_scan_kernels(dt, counts, heads, groups, N, P, taps):
+def test_conv_and_scan_kernels(dt, rate, counts, heads, groups, N, P, taps):
     """The convolution and the scan against their plain torch references, from states that are not zero, in slots that are
-    not the sequences' numbers."""
+    not the sequences' numbers.  rate: added to A_log; decays of e^-12 and e^-55 a row and less, whose running product
+    leaves float32's range within a few rows, or which do so alone."""
     ops = Runtime(dtype="float32", device=DEV).ops
     m, inner, n = sum(counts), heads * P, len(counts)
     C = inner + 2 * groups * N
@@ -224,7 +226,7 @@ def test_conv_and_scan_kernels(dt, counts, heads, groups, N, P, taps):
     row_seq = torch.repeat_interleave(torch.arange(n, dtype=torch.int32), torch.tensor(counts))
     cst = rnd(7, max(taps - 1, 1), C, seed=4)[:, :taps - 1].contiguous() if taps > 1 else None
     sst = rnd(7, heads, N, P, seed=5)
-    dt_bias, a_log, skip = rnd(heads, seed=6), rnd(heads, seed=7, scale=0.5), 1 + rnd(heads, seed=8, scale=0.2)
+    dt_bias, a_log, skip = rnd(heads, seed=6), rnd(heads, seed=7, scale=0.5) + rate, 1 + rnd(heads, seed=8, scale=0.2)
     cst_r, sst_r = (cst.clone() if cst is not None else None), sst.clone()
     xbc_r = ref_ops.conv_act(u[:, inner:inner + C], wt, bias, cst_r, slots, cu, row_seq, "silu")
     y_r = ref_ops.ssd_scan(xbc_r, u[:, :inner], u[:, inner + C:], dt_bias, a_log, skip, sst_r, slots, cu, max(counts), heads, groups, N, P)
@@ -235,7 +237,7 @@ def test_conv_and_scan_kernels(dt, counts, heads, groups, N, P, taps):
                      max(counts), heads, groups, N, P)
     assert rel_l2(xbc, xbc_r) < (2e-6 if dt == torch.float32 else 4e-3)
     assert cst is None or torch.equal(cst_d.cpu(), cst_r)
-    assert rel_l2(y, y_r) < 3e-6 and rel_l2(sst_d, sst_r) < 1e-6
+    assert rel_l2(y, y_r) < 3e-6 and rel_l2(sst_d, sst_r) < 2e-6 and bool(torch.isfinite(y).all()) and bool(torch.isfinite(sst_d).all())
     untouched = [s for s in range(7) if s not in slots.tolist()]
     assert torch.equal(sst_d[untouched].cpu(), sst[untouched])
 

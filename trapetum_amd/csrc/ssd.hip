@@ -173,7 +173,7 @@ ssd_scan_k(SsdArgs a) {
     constexpr int TC = 16 / R, NQ = NR / 4, PAIRS = TC * R;        // PAIRS = 16 (row, unit) pairs a round
     constexpr int J = (TC * NR / VEC + 255) / 256;       // packs of B (and of C) a thread stages a round
     using Pk = Pack<T, VEC>;
-    extern __shared__ float lds[];                       // B [TC][NR], C [TC][NR], dt [PAIRS], decay [PAIRS], x [PAIRS][64], z [PAIRS][64], parts [4][PAIRS][64]
+    extern __shared__ __attribute__((aligned(16))) float lds[];      // B [TC][NR], C [TC][NR], dt [PAIRS], decay [PAIRS], x [PAIRS][64], z [PAIRS][64], parts [4][PAIRS][64]
     const int seq = blockIdx.x, tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
     const int N = a.N, P = a.P, hpg = a.heads / a.groups, pcs = (P + 63) / 64, units = hpg * pcs, bpg = (units + R - 1) / R;
     const int g = blockIdx.y / bpg, u0 = (blockIdx.y - g * bpg) * R;
@@ -285,14 +285,21 @@ ssd_scan_k(SsdArgs a) {
                 dx[r] = dts[t * R + r] * xs[(t * R + r) * 64 + lane];
                 acc[r] = 0.f;
             }
-            const float* Bt = Bs + t * NR + n0; const float* Ct = Cs + t * NR + n0;
+            // four neighbouring elements of B and of C a read (rows start on 16 bytes: NR and a wave's first row are multiples of 4)
+            const float4* Bt = reinterpret_cast<const float4*>(Bs + t * NR + n0);
+            const float4* Ct = reinterpret_cast<const float4*>(Cs + t * NR + n0);
 #pragma unroll
-            for (int n = 0; n < NQ; n++) {
-                const float bn = Bt[n], cn = Ct[n];
+            for (int n4 = 0; n4 < NQ / 4; n4++) {
+                const float4 b4 = Bt[n4], c4 = Ct[n4];
+                const float bn[4] = {b4.x, b4.y, b4.z, b4.w}, cn[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
-                for (int r = 0; r < R; r++) {
-                    S[r][n] = __builtin_fmaf(d[r], S[r][n], dx[r] * bn);
-                    if (MODE != 1) acc[r] = __builtin_fmaf(S[r][n], cn, acc[r]);
+                for (int e = 0; e < 4; e++) {
+                    const int n = 4 * n4 + e;
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        S[r][n] = __builtin_fmaf(d[r], S[r][n], dx[r] * bn[e]);
+                        if (MODE != 1) acc[r] = __builtin_fmaf(S[r][n], cn[e], acc[r]);
+                    }
                 }
             }
 #pragma unroll
@@ -355,8 +362,8 @@ ssd_carry_k(SsdArgs a) {
 }
 
 // Units of 64 channels a block takes.  Two (where a group of heads has two), which halves the reads of B and C from LDS,
-// measured the same as one (217 against 219 us for 2,048 rows of 36 heads x 64 channels with a state of 128) at fewer waves
-// a SIMD: the kernel keeps the parameter, one unit is what is compiled.
+// measured slower than one (209 against 170 us for 2,048 rows of 36 heads x 64 channels with a state of 128; a decode step
+// 9.2 against 8.2): the kernel keeps the parameter, one unit is what is compiled.
 static int scan_units(const SsdArgs&) { return 1; }
 static int scan_nr(int N) { return N <= 16 ? 16 : N <= 32 ? 32 : N <= 64 ? 64 : N <= 128 ? 128 : 256; }
 static size_t scan_lds(int N) { return (size_t)(2 * 16 * scan_nr(N) + 32 + 6 * 16 * 64) * sizeof(float); }     // 16 rows x 1 unit, or 8 x 2
